@@ -47,6 +47,37 @@ class BlockPool:
         return (num_tokens + self.block_size - 1) // self.block_size
 
 
+class StateSlotPool:
+    """Fixed-size recurrent-state slots, one per live sequence, for models
+    whose mixers carry per-sequence state (linear recurrences, short
+    convolution tails) beside or instead of paged K/V. A slot is taken at
+    admission and returned at finish or preemption; its content is never
+    cleared on the host — the kernels treat a chunk that starts at
+    position 0 as starting from the zero state, whatever the slot held."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free: List[int] = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def can_allocate(self) -> bool:
+        return bool(self._free)
+
+    def allocate(self) -> int:
+        if not self._free:
+            raise RuntimeError("state slots exhausted")
+        return self._free.pop()
+
+    def free(self, slot: int) -> None:
+        if slot < 0:
+            return
+        assert slot not in self._free, f"state slot {slot} freed twice"
+        self._free.append(slot)
+
+
 class PrefixCachingPool(BlockPool):
     """Block-hash automatic prefix caching (the vLLM-APC analog the
     reference gets from its vLLM backend). Full prompt blocks are

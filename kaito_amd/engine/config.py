@@ -75,6 +75,9 @@ class ModelConfig:
     # routing: "softmax_topk" (mixtral: softmax→topk→renorm) |
     # "topk_softmax" (gpt-oss: topk logits→softmax over the k)
     moe_routing: str = "softmax_topk"
+    # router logits in f32 (x and the router matrix are widened before the
+    # product) instead of the activation dtype
+    moe_router_fp32: bool = False
     # attention scale override (padded-head models: phi-2 pads 80→128 for
     # the D∈{64,128,256} kernels but keeps 80^-0.5 scaling; zero-padded
     # dims contribute nothing, so the math is exact)
@@ -114,6 +117,20 @@ class ModelConfig:
     # "transformers" → fallback runtime (reference: vLLM vs text-generation
     # runtime split, supported_models.yaml `runtime:` field)
     runtime: str = "native"
+    # ---- model class + heterogeneous layer stacks -----------------------
+    # which model class serves this config (models/registry.py
+    # MODEL_CLASSES): "llama" covers every homogeneous transformer above;
+    # "gurapel" is the hybrid stack described by `layer_specs`
+    arch: str = "llama"
+    # one LayerSpec per layer (models/hybrid_config.py) for stacks whose
+    # layers differ in kind (recurrent / windowed attention / parallel
+    # pairs); None for homogeneous models
+    layer_specs: Optional[tuple] = None
+    # learned absolute position table added to the scaled embedding
+    learned_positions: bool = False
+    # the residual stream is held and summed in f32 (norms read it in
+    # f32); sub-layers see its rounding to `dtype`
+    residual_fp32: bool = False
 
     @classmethod
     def from_hf_config(cls, cfg: dict, name: str = "") -> "ModelConfig":

@@ -61,6 +61,14 @@ class LLMEngine:
         self.runner = ModelRunner(cfg).load_model(weights_path, cfg.seed)
         self.runner.setup_tunable()
         self.runner.profile_and_allocate_kv()
+        self.state_pool = None
+        if self.runner.stateful:
+            # a cached K/V prefix cannot restore a recurrent state, and the
+            # host offload store knows only K/V pages
+            cfg.enable_prefix_caching = False
+            cfg.kv_offload = False
+            from .block_pool import StateSlotPool
+            self.state_pool = StateSlotPool(self.runner.num_state_slots)
         if cfg.enable_prefix_caching:
             from .block_pool import PrefixCachingPool
             self.pool = PrefixCachingPool(self.runner.num_gpu_blocks,
@@ -77,7 +85,8 @@ class LLMEngine:
         if self.kv_offload is not None:
             restore_cb = lambda seq: self.kv_offload.restore_prefix(  # noqa: E731
                 seq.prompt_token_ids, seq.block_table)
-        self.scheduler = Scheduler(cfg, self.pool, restore_cb)
+        self.scheduler = Scheduler(cfg, self.pool, restore_cb,
+                                   state_pool=self.state_pool)
         self.sampler = Sampler(cfg.device, cfg.seed)
         from ..parallel.state import get_state
         self._pp = get_state().pp_size > 1
@@ -534,6 +543,61 @@ class LLMEngine:
                 self.scheduler.finish(seq)
                 finished.append(seq)
         return finished
+
+    # ------------------------------------------------- externally driven
+    #
+    # A caller that owns the schedule (trace replay, conformance runs)
+    # composes each step itself: which requests advance, by how many of
+    # their known tokens, and at which rows it wants logits. Everything
+    # below the composition is the serving path: the scheduler's
+    # admission / page growth / release, the runner's batch preparation
+    # and the model's kernels. Nothing is sampled.
+    def extend_request(self, seq_id: int, tokens: List[int]) -> None:
+        """Append known tokens to a request (created on first use)."""
+        seq = self.seqs.get(seq_id)
+        if seq is None:
+            seq = Sequence(seq_id, [], SamplingParams(max_tokens=0))
+            self.seqs[seq_id] = seq
+            self.scheduler.add(seq)
+        seq.prompt_token_ids.extend(int(t) for t in tokens)
+        if seq.num_tokens > self.runner.max_model_len:
+            raise ValueError(
+                f"request {seq_id} exceeds max_model_len="
+                f"{self.runner.max_model_len}")
+
+    @torch.no_grad()
+    def step_explicit(self, portions, want) -> Optional[torch.Tensor]:
+        """Run ONE batch of (seq_id, n_tokens) portions — the next n known
+        tokens of each request, prompt-sized or single — and return f32
+        logits [len(want), vocab] at `want` = [(portion_index,
+        offset_in_portion)], in that order (None if nothing is wanted)."""
+        self.flush()
+        batch = self.scheduler.schedule_explicit(
+            [(self.seqs[sid], n) for sid, n in portions])
+        base, acc = [], 0
+        for c in batch.chunks:
+            base.append(acc)
+            acc += c.length
+        rows = [base[i] + off for i, off in want]
+        hidden = self.runner.execute_prefill(batch.chunks, rows=rows)
+        self.scheduler.advance_prefill_chunks(batch)
+        for c in batch.chunks:
+            c.seq.sched_len = c.seq.prefilled_len
+        if not rows:
+            return None
+        return self.runner.model.compute_logits(hidden).float()
+
+    def release(self, seq_id: int) -> None:
+        """End a request: its pages and state slot return to the pools."""
+        seq = self.seqs.pop(seq_id, None)
+        if seq is None:
+            return
+        if seq.status == SeqStatus.RUNNING:
+            self.scheduler.finish(seq)
+        elif seq in self.scheduler.waiting:
+            self.scheduler.waiting.remove(seq)
+        seq.status = SeqStatus.FINISHED
+        seq.finish_reason = "released"
 
     # ------------------------------------------------------------- offline
     def generate(self, prompts: List[List[int]],

@@ -210,7 +210,7 @@ class LoRAManager:
         T = x.size(0)
         if x.is_cuda:
             from .. import ops
-            ops.load_extension()
+            ops.load_extension("quant")
             tmp = torch.empty(T, R, dtype=torch.float32, device=x.device)
             # per-adapter alpha/r scaling is folded into A at registration
             torch.ops.kaito.lora_shrink(tmp, x, A, ids, 1.0)

@@ -25,7 +25,8 @@ from .config import EngineConfig
 from .scheduler import ScheduledBatch
 from .sequence import Sequence
 from . import lora as lora_mod
-from ..models.llama import AttnMetadata, LlamaForCausalLM
+from ..models.llama import AttnMetadata
+from ..models.registry import resolve_model_class
 from ..parallel import state as ps
 
 logger = logging.getLogger(__name__)
@@ -37,7 +38,12 @@ class ModelRunner:
         self.device = torch.device(cfg.device)
         self.is_gpu = self.device.type == "cuda"
         torch.manual_seed(cfg.seed)
-        self.model = LlamaForCausalLM(cfg.model).to(self.device)
+        self.model = resolve_model_class(cfg.model)(cfg.model).to(self.device)
+        # models whose mixers carry per-sequence recurrent state: the
+        # runner sizes a slot per live sequence and always hands the
+        # model the unified chunk metadata (no fresh-prompt fast path)
+        self.stateful = bool(getattr(self.model, "uses_state_slots", False))
+        self.num_state_slots = 0
         self.kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = []
         self.num_gpu_blocks = 0
         self.max_model_len = cfg.max_model_len or cfg.model.max_position
@@ -82,6 +88,8 @@ class ModelRunner:
         """Size the KV pool from free VRAM (auto max-model-len semantics)."""
         cfg = self.cfg
         m = cfg.model
+        if self.stateful:
+            return self._allocate_hybrid_caches()
         tp = max(cfg.tensor_parallel_size, 1)
         kvh = max(m.num_kv_heads // tp, 1)
         fp8 = cfg.kv_cache_dtype == "fp8"
@@ -135,6 +143,36 @@ class ModelRunner:
                     n_blocks * block_bytes / (1 << 30))
         return n_blocks
 
+    def _allocate_hybrid_caches(self) -> int:
+        """Hybrid stacks: the model states what each layer keeps — K/V
+        pages for its attention mixers, one state slot per live sequence
+        for its recurrent mixers. Slots are sized by max_num_seqs first;
+        pages take the rest of the budget."""
+        cfg = self.cfg
+        if cfg.kv_cache_dtype == "fp8":
+            raise ValueError("fp8 KV cache not supported for hybrid stacks")
+        page_bytes, slot_bytes = self.model.cache_bytes(cfg.block_size)
+        n_slots = cfg.max_num_seqs
+        if cfg.num_gpu_blocks is not None:
+            n_blocks = cfg.num_gpu_blocks
+        elif self.is_gpu and page_bytes > 0:
+            free, total = torch.cuda.mem_get_info(self.device)
+            budget = int(total * cfg.gpu_memory_utilization) \
+                - (total - free) - n_slots * slot_bytes
+            n_blocks = max(budget // page_bytes, 16)
+        else:
+            n_blocks = 512
+        cap = cfg.max_num_seqs * cfg.max_blocks_per_seq(self.max_model_len) + 1
+        n_blocks = min(n_blocks, cap)
+        self.num_gpu_blocks = n_blocks
+        self.num_state_slots = n_slots
+        self.kv_caches = self.model.alloc_caches(
+            n_blocks, cfg.block_size, n_slots, self.device)
+        logger.info("hybrid caches: %d pages (%.2f GiB), %d state slots "
+                    "(%.2f GiB)", n_blocks, n_blocks * page_bytes / (1 << 30),
+                    n_slots, n_slots * slot_bytes / (1 << 30))
+        return n_blocks
+
     # ------------------------------------------------------------- helpers
     def _slot(self, seq: Sequence, pos: int) -> int:
         bs = self.cfg.block_size
@@ -142,14 +180,17 @@ class ModelRunner:
 
     # ------------------------------------------------------------- prefill
     @torch.no_grad()
-    def execute_prefill(self, chunks) -> torch.Tensor:
+    def execute_prefill(self, chunks, rows=None) -> torch.Tensor:
         """Run a (possibly chunked) prefill batch. Each chunk covers prompt
         tokens [start, start+length) of its sequence; chunks with start>0
         or incomplete prompts use context attention over the paged cache.
         Returns hidden states of the LAST token of each COMPLETING chunk,
-        in chunk order (aligned with batch.sampling_seqs)."""
+        in chunk order (aligned with batch.sampling_seqs) — or, with
+        `rows` (indices into the concatenated chunk rows), of exactly
+        those rows."""
         ids, pos, slots, cu = [], [], [], [0]
-        fresh = all(c.start == 0 and c.completes for c in chunks)
+        fresh = (not self.stateful
+                 and all(c.start == 0 and c.completes for c in chunks))
         for c in chunks:
             toks = c.seq.context_token_ids[c.start:c.start + c.length]
             ids.extend(toks)
@@ -178,6 +219,17 @@ class ModelRunner:
             max_seqlen=max(c.length for c in chunks),
             block_tables=block_tables,
             kv_lens=kv_lens)
+        if self.stateful:
+            seq_of = []
+            for i, c in enumerate(chunks):
+                seq_of.extend([i] * c.length)
+            meta.state_slots = torch.tensor(
+                [c.seq.state_slot for c in chunks], dtype=torch.int32,
+                device=dev)
+            meta.seq_starts = torch.tensor(
+                [c.start for c in chunks], dtype=torch.int32, device=dev)
+            meta.token_seq = torch.tensor(seq_of, dtype=torch.int32,
+                                          device=dev)
         if self.lora_manager is not None:
             tok_ids = []
             for c in chunks:
@@ -189,7 +241,8 @@ class ModelRunner:
             lora_mod.set_active(None, None)
         if hidden is None:
             return None  # intermediate PP stage
-        last = [cu[i + 1] - 1 for i, c in enumerate(chunks) if c.completes]
+        last = [cu[i + 1] - 1 for i, c in enumerate(chunks) if c.completes] \
+            if rows is None else list(rows)
         if not last:
             return hidden[:0]
         return hidden[torch.tensor(last, device=dev)]
@@ -208,6 +261,19 @@ class ModelRunner:
             "seq_lens": torch.zeros(max_bs, dtype=torch.int32, device=dev),
             "lora_ids": torch.full((max_bs,), -1, dtype=torch.int32, device=dev),
         }
+        if self.stateful:
+            # decode = chunks of one token: static layout tensors, plus
+            # the per-sequence slot (-1 pads) and start position
+            self._buf.update({
+                "state_slots": torch.full((max_bs,), -1, dtype=torch.int32,
+                                          device=dev),
+                "seq_starts": torch.zeros(max_bs, dtype=torch.int32,
+                                          device=dev),
+                "cu_seqlens": torch.arange(max_bs + 1, dtype=torch.int32,
+                                           device=dev),
+                "token_seq": torch.arange(max_bs, dtype=torch.int32,
+                                          device=dev),
+            })
         self._max_blocks = mb
 
     def _model_forward(self, input_ids, positions, meta):
@@ -239,6 +305,11 @@ class ModelRunner:
             slot_mapping=b["slot_mapping"][:bs],
             block_tables=b["block_tables"][:bs],
             seq_lens=b["seq_lens"][:bs])
+        if self.stateful:
+            meta.cu_seqlens = b["cu_seqlens"][:bs + 1]
+            meta.state_slots = b["state_slots"][:bs]
+            meta.seq_starts = b["seq_starts"][:bs]
+            meta.token_seq = b["token_seq"][:bs]
         return self._model_forward(b["input_ids"][:bs], b["positions"][:bs],
                                    meta)
 
@@ -314,8 +385,14 @@ class ModelRunner:
         ie = m.moe_intermediate_size or m.intermediate_size
         ie_local = ie if (tp > 1 and m.num_experts % tp == 0) or tp == 1 \
             else ie // tp   # mirrors MoEMLP's EP-vs-IE sharding choice
-        if m.num_experts > 0 and (m.hidden_size % 64 != 0 or
-                                  ie_local % 64 != 0):
+        capturable = getattr(self.model, "decode_graph_capturable", None)
+        if capturable is not None:
+            if not capturable():
+                logger.info("model has host-synchronising decode ops: "
+                            "skipping decode graph capture")
+                return
+        elif m.num_experts > 0 and (m.hidden_size % 64 != 0 or
+                                    ie_local % 64 != 0):
             # odd shapes fall back to the per-expert torch loop, whose
             # host-side segment reads cannot be captured
             logger.info("MoE model with non-64-aligned dims: "
@@ -324,6 +401,10 @@ class ModelRunner:
         if not hasattr(self, "_buf"):
             self._init_decode_buffers()
         self._buf["seq_lens"].fill_(1)  # benign shapes for capture
+        if self.stateful:
+            # warm-up and capture passes must not advance any sequence's
+            # recurrent state: every row is a padding row (slot -1)
+            self._buf["state_slots"].fill_(-1)
         torch.cuda.synchronize()
         for bs in sorted(self.cfg.graph_batch_sizes, reverse=True):
             if bs > self.cfg.max_num_seqs:
@@ -375,6 +456,8 @@ class ModelRunner:
             b["input_ids"][:bs].copy_(sampled[:bs])
             b["positions"][:bs] += 1
             b["seq_lens"][:bs] += 1
+            if self.stateful:
+                b["seq_starts"][:bs] += 1
             for i, s in enumerate(seqs):
                 if getattr(s, "_bt_dirty", False):
                     n = len(s.block_table)
@@ -413,6 +496,12 @@ class ModelRunner:
                 torch.tensor(slots, dtype=torch.long), non_blocking=True)
             b["seq_lens"][:bs].copy_(
                 torch.tensor(lens, dtype=torch.int32), non_blocking=True)
+            if self.stateful:
+                b["state_slots"][:bs].copy_(torch.tensor(
+                    [s.state_slot for s in seqs], dtype=torch.int32),
+                    non_blocking=True)
+                b["seq_starts"][:bs].copy_(
+                    torch.tensor(pos, dtype=torch.int32), non_blocking=True)
             import numpy as np
             flat = np.zeros((bs, self._max_blocks), dtype=np.int32)
             for i, s in enumerate(seqs):
@@ -432,6 +521,8 @@ class ModelRunner:
             if bucket > bs:
                 b["seq_lens"][bs:bucket].zero_()
                 b["slot_mapping"][bs:bucket].fill_(-1)
+                if self.stateful:
+                    b["state_slots"][bs:bucket].fill_(-1)
             g, out = self._graphs[bucket]
             g.replay()
             return out[:bs]

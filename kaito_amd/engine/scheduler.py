@@ -57,9 +57,12 @@ class ScheduledBatch:
 
 class Scheduler:
     def __init__(self, cfg: EngineConfig, pool: BlockPool,
-                 restore_cb=None):
+                 restore_cb=None, state_pool=None):
         self.cfg = cfg
         self.pool = pool
+        # recurrent-state slots (StateSlotPool) for models that carry
+        # per-sequence state; None for pure paged-KV models
+        self.state_pool = state_pool
         self.waiting: deque[Sequence] = deque()
         self.prefilling: List[Sequence] = []   # admitted, prompt KV partial
         self.running: List[Sequence] = []
@@ -138,6 +141,10 @@ class Scheduler:
             need = self.pool.blocks_needed(seq.num_tokens + 1)
             if not self.pool.can_allocate(need):
                 break
+            if self.state_pool is not None:
+                if not self.state_pool.can_allocate():
+                    break
+                seq.state_slot = self.state_pool.allocate()
             self.waiting.popleft()
             shared = []
             if hasattr(self.pool, "match_prefix"):
@@ -162,6 +169,7 @@ class Scheduler:
                 # put it back; it needs a step with a larger free budget
                 self.waiting.appendleft(seq)
                 self.pool.free(seq.block_table)
+                self._free_state(seq)
                 seq.block_table = []
                 seq.status = SeqStatus.WAITING
                 break
@@ -218,6 +226,7 @@ class Scheduler:
                     victim = batch.pop()  # newest scheduled
                     self.running.remove(victim)
                     self.pool.free(victim.block_table)
+                    self._free_state(victim)   # recomputed from position 0
                     # recompute preemption (vLLM semantics): KEEP the
                     # generated tokens — they were already streamed to the
                     # client — and re-prefill prompt+generated as context
@@ -234,8 +243,46 @@ class Scheduler:
             return None
         return ScheduledBatch(is_prefill=False, seqs=batch)
 
+    def _free_state(self, seq: Sequence) -> None:
+        if self.state_pool is not None and seq.state_slot >= 0:
+            self.state_pool.free(seq.state_slot)
+        seq.state_slot = -1
+
+    # ---- externally composed steps (trace replay) ----
+    def schedule_explicit(self, portions) -> ScheduledBatch:
+        """Build ONE batch from a caller-composed list of
+        (seq, n_new_tokens): the next n tokens of seq's known context,
+        decode-sized or prompt-sized alike. A sequence is admitted (state
+        slot taken) at its first portion; pages are taken as the tokens
+        arrive rather than for a whole prompt upfront, since the caller
+        may not know the final length. Raises if pages or slots run out —
+        the caller composed the step, so there is nobody to preempt."""
+        chunks: List[PrefillChunk] = []
+        for seq, n in portions:
+            if seq.status == SeqStatus.WAITING:
+                if seq in self.waiting:
+                    self.waiting.remove(seq)
+                if self.state_pool is not None:
+                    seq.state_slot = self.state_pool.allocate()
+                seq.status = SeqStatus.RUNNING
+                self.prefilling.append(seq)
+            start = seq.prefilled_len
+            if n <= 0 or start + n > seq.num_context_tokens:
+                raise ValueError(
+                    f"portion [{start}, {start + n}) outside the "
+                    f"{seq.num_context_tokens} known tokens of seq "
+                    f"{seq.seq_id}")
+            need = self.pool.blocks_needed(start + n) - len(seq.block_table)
+            if need > 0:
+                seq.block_table.extend(self.pool.allocate(need))
+                seq._bt_dirty = True
+            chunks.append(PrefillChunk(seq, start, n))
+        return ScheduledBatch(is_prefill=True,
+                              seqs=[c.seq for c in chunks], chunks=chunks)
+
     def finish(self, seq: Sequence) -> None:
         self.pool.free(seq.block_table)
+        self._free_state(seq)
         seq.block_table = []
         if seq in self.running:
             self.running.remove(seq)

@@ -56,6 +56,8 @@ class Sequence:
     # bumped on preemption so stale in-flight results are dropped at resolve
     epoch: int = 0
     lora_id: int = -1            # adapter slot (-1 = base model)
+    # recurrent-state slot (models with per-sequence state; -1 = none)
+    state_slot: int = -1
     # prompt tokens whose KV is in the cache (chunked prefill / prefix
     # restore); prompt fully prefilled when == num_prompt_tokens
     prefilled_len: int = 0

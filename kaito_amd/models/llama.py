@@ -39,6 +39,11 @@ class AttnMetadata:
     # context-prefill (chunked prefill / prefix-cache continuation):
     # q covers only suffix tokens; K/V read from the paged cache.
     kv_lens: Optional[torch.Tensor] = None       # [B] int32 total ctx len
+    # models with per-sequence recurrent state (every step, decode too, is
+    # a list of chunks: cu_seqlens delimits them):
+    state_slots: Optional[torch.Tensor] = None   # [B] int32, <0 = padding
+    seq_starts: Optional[torch.Tensor] = None    # [B] int32 first position
+    token_seq: Optional[torch.Tensor] = None     # [T] int32 chunk of a row
 
 
 def build_cos_sin_cache(cfg: ModelConfig, device, max_pos: Optional[int] = None,

@@ -24,6 +24,8 @@ def _shard(t: torch.Tensor, dim: int) -> torch.Tensor:
 
 def load_safetensors_weights(model, path: str,
                              skip_projections: bool = False) -> None:
+    if getattr(model.cfg, "arch", "llama") == "gurapel":
+        return load_gurapel_weights(model, path)
     from safetensors.torch import safe_open
 
     cfg = model.cfg
@@ -244,3 +246,101 @@ def load_safetensors_weights(model, path: str,
                         torch.cat([w1, w3], 0).to(moe.dtype))
                     params[pre + "mlp.w_down"][le].copy_(
                         get(ex + "w2.weight").to(moe.dtype))
+
+
+# ---- hybrid stacks ------------------------------------------------------
+
+def load_gurapel_weights(model, path: str) -> None:
+    """Gurapel checkpoint (flat tensor names, `l<i>.` per layer, linear
+    weights [out, in]) → GurapelForCausalLM. Fuses the per-mixer input
+    projections, folds the one-plus norm weights and the recurrence's
+    decay constant, and widens every small per-channel tensor to f32."""
+    from safetensors.torch import safe_open
+
+    tensors: Dict[str, torch.Tensor] = {}
+    for f in sorted(Path(path).glob("*.safetensors")):
+        with safe_open(str(f), framework="pt", device="cpu") as sf:
+            for k in sf.keys():
+                tensors[k] = sf.get_tensor(k)
+    if not tensors:
+        raise FileNotFoundError(f"no safetensors under {path}")
+    cfg = model.cfg
+    used = set()
+
+    def get(name):
+        used.add(name)
+        return tensors[name]
+
+    def put(param, value):
+        if tuple(param.shape) != tuple(value.shape):
+            raise ValueError(f"shape mismatch: parameter {tuple(param.shape)}"
+                             f" vs checkpoint {tuple(value.shape)}")
+        with torch.no_grad():
+            param.copy_(value.to(param.dtype))
+
+    def one_plus(name):
+        return get(name).float() + 1.0
+
+    put(model.embed_tokens.weight, get("embed"))
+    put(model.pos_embed, get("pos"))
+    put(model.norm, one_plus("final.norm"))
+    put(model.lm_head, get("head"))
+    for i, layer in enumerate(model.layers):
+        pre = f"l{i}."
+        spec = layer.spec
+        put(layer.norm1, one_plus(pre + "norm1"))
+        if spec.kind == "delta":
+            m, mp = layer.mixer, pre + "mix."
+            put(m.in_proj, torch.cat(
+                [get(mp + n) for n in ("q", "k", "v", "g", "a", "b")], 0))
+            put(m.conv_weight, torch.cat(
+                [get(mp + n + ".conv") for n in ("q", "k", "v")], 0).float())
+            put(m.a_log, get(mp + "A_log").float())
+            put(m.dt_bias, get(mp + "dt_bias").float())
+            put(m.out_norm, get(mp + "norm").float())
+            put(m.o_proj, get(mp + "o"))
+        else:
+            a, ap = layer.attn, pre + "mix.left."
+            put(a.qkv_proj, torch.cat(
+                [get(ap + n) for n in ("q", "k", "v")], 0))
+            put(a.q_norm, get(ap + "q.norm").float())
+            put(a.k_norm, get(ap + "k.norm").float())
+            put(a.r1, get(ap + "r1").float())
+            put(a.r2, get(ap + "r2").float())
+            put(a.o_proj, get(ap + "o"))
+            r, rp = layer.rglru, pre + "mix.right."
+            put(r.in_proj, torch.cat([get(rp + "y"), get(rp + "x")], 0))
+            put(r.in_bias, torch.cat([get(rp + "y.b"), get(rp + "x.b")], 0))
+            put(r.conv_weight, get(rp + "conv").float())
+            put(r.conv_bias, get(rp + "conv.b").float())
+            # [blocks, out, in] ×2 → [blocks, in, 2·out]
+            put(r.gate_w, torch.cat(
+                [get(rp + "ra").float().transpose(1, 2),
+                 get(rp + "ri").float().transpose(1, 2)], 2))
+            put(r.gate_b, torch.cat(
+                [get(rp + "ra.b").float(), get(rp + "ri.b").float()],
+                1).unsqueeze(1))
+            put(r.decay_rate, r.spec.decay_scale *
+                torch.nn.functional.softplus(get(rp + "lam").float()))
+            put(r.o_proj, get(rp + "o"))
+            put(layer.attn_out_norm, get(pre + "mix.left.out").float())
+            put(layer.rglru_out_norm, get(pre + "mix.right.out").float())
+        if layer.mlp is not None:
+            mlp, fp = layer.mlp, pre + "mlp."
+            put(layer.norm2, one_plus(pre + "norm2"))
+            put(mlp.gate, get(fp + "router").float())
+            ie = mlp.ie_local
+            with torch.no_grad():
+                mlp.w_gate_up.zero_()
+                mlp.w_down.zero_()
+                for e in range(mlp.num_experts):
+                    g, u, d = (get(f"{fp}e{e}.{n}")
+                               for n in ("gate", "up", "down"))
+                    ff = g.shape[0]
+                    mlp.w_gate_up[e, :ff].copy_(g.to(mlp.w_gate_up.dtype))
+                    mlp.w_gate_up[e, ie:ie + ff].copy_(
+                        u.to(mlp.w_gate_up.dtype))
+                    mlp.w_down[e, :, :ff].copy_(d.to(mlp.w_down.dtype))
+    extra = set(tensors) - used
+    if extra:
+        raise ValueError(f"unused checkpoint tensors: {sorted(extra)[:8]}")

@@ -50,8 +50,12 @@ class MoEMLP(nn.Module):
             self.e_local = e
             self.e_base = 0
             self.ie_local = ie // tp
-        self.gate = nn.Parameter(torch.empty(e, h, dtype=cfg.dtype),
-                                 requires_grad=False)
+        # f32 router option: the matrix is held in f32 and x is widened
+        # before the product, so no logit is rounded to the activation
+        # dtype before top-k
+        self.gate = nn.Parameter(
+            torch.empty(e, h, dtype=torch.float32 if cfg.moe_router_fp32
+                        else cfg.dtype), requires_grad=False)
         # stacked expert weights (local shard):
         # [E_l, 2*IE_l, h] (gate|up) and [E_l, h, IE_l]
         self.w_gate_up = nn.Parameter(
@@ -96,7 +100,10 @@ class MoEMLP(nn.Module):
         (sorted_tok int32 [TK], gates f32 [TK], offsets int32 [E+1])."""
         T = x.size(0)
         cfg = self.cfg
-        logits = torch.nn.functional.linear(x, self.gate)      # [T, E]
+        if cfg.moe_router_fp32:
+            logits = torch.nn.functional.linear(x.float(), self.gate)
+        else:
+            logits = torch.nn.functional.linear(x, self.gate)  # [T, E]
         if cfg.moe_routing == "noaux_tc":
             # deepseek-v3: sigmoid scores; SELECTION uses scores+bias with
             # group-limited top-k; WEIGHTS are the original sigmoid scores
@@ -156,7 +163,8 @@ class MoEMLP(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         T, H = x.shape
         sorted_tok, gates, offsets = self._route(x)
-        fused_shapes = x.is_cuda and H % 64 == 0 and self.ie_local % 64 == 0
+        fused_shapes = (x.is_cuda and x.dtype == torch.bfloat16
+                        and H % 64 == 0 and self.ie_local % 64 == 0)
         # under hipGraph capture the fused kernels are mandatory (the
         # per-expert loop reads segment sizes on the host): deepseek k=6
         # crosses TK=4096 at decode bs>682 and measured 30.9k vs timeout

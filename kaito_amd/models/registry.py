@@ -19,6 +19,39 @@ def register(cfg: ModelConfig) -> ModelConfig:
     return cfg
 
 
+# arch → "module:class" of the model class that serves it (resolved lazily
+# so importing the catalog stays cheap)
+MODEL_CLASSES: Dict[str, str] = {
+    "llama": "kaito_amd.models.llama:LlamaForCausalLM",
+    "gurapel": "kaito_amd.models.gurapel:GurapelForCausalLM",
+}
+
+
+def resolve_model_class(cfg: ModelConfig):
+    import importlib
+    try:
+        mod, cls = MODEL_CLASSES[cfg.arch].split(":")
+    except KeyError:
+        raise KeyError(f"no model class for arch {cfg.arch!r}; known: "
+                       f"{sorted(MODEL_CLASSES)}") from None
+    return getattr(importlib.import_module(mod), cls)
+
+
+def config_from_checkpoint(cfg_json: dict, name: str = "",
+                           dtype=None) -> ModelConfig:
+    """config.json dict → ModelConfig, choosing the reader by the file's
+    own architecture tag."""
+    from .hybrid_config import gurapel_model_config, is_gurapel_config
+    if is_gurapel_config(cfg_json):
+        kw = {"dtype": dtype} if dtype is not None else {}
+        return gurapel_model_config(cfg_json, name=name, **kw)
+    cfg = ModelConfig.from_hf_config(cfg_json, name=name)
+    if dtype is not None:
+        import dataclasses
+        cfg = dataclasses.replace(cfg, dtype=dtype)
+    return cfg
+
+
 def get_model_config(name: str, weights_path: str = None) -> ModelConfig:
     """Resolve a preset by name; unknown names fall back to dynamic
     resolution from the weights directory's config.json (the reference's
@@ -33,7 +66,7 @@ def get_model_config(name: str, weights_path: str = None) -> ModelConfig:
         cfg_path = os.path.join(weights_path, "config.json")
         if os.path.exists(cfg_path):
             with open(cfg_path) as f:
-                cfg = ModelConfig.from_hf_config(json.load(f), name=name)
+                cfg = config_from_checkpoint(json.load(f), name=name)
             return register(cfg)
     raise KeyError(f"unknown model preset: {name}; known: {sorted(_REGISTRY)}")
 

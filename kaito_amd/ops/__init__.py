@@ -5,48 +5,92 @@ Dispatch policy (engine contract):
     missing on a GPU machine this raises loudly — there is NO silent
     eager fallback on GPU.
   * CPU tensors → torch_ref reference implementations (tests / no-GPU dev).
+
+The extension is split into kernel groups (ops/_build.py GROUPS), one
+shared library each; a group is built (if absent) and loaded the first
+time one of its ops is called.
 """
 from __future__ import annotations
 
 import torch
 
 from . import torch_ref
-from ._build import SO_PATH
+from ._build import GROUPS, SO_PATH, so_path
 
-_LOADED = False
+_LOADED: set = set()
+
+# op name → kernel group that registers it
+_OP_GROUP = {}
+for _g, _names in {
+    "core": ("rms_norm fused_add_rms_norm rotary_embedding silu_and_mul "
+             "gelu_and_mul gelu layer_norm fused_add_layer_norm "
+             "reshape_and_cache topk"),
+    "attn": ("paged_attention paged_attention_sp prefill_attention "
+             "context_attention mfma_tile_gemm paged_read_bw"),
+    "mla": "mla_decode mla_cache_write",
+    "moe": "moe_gate_silu moe_down_scatter",
+    "quant": "w4a16_gemv w4a16_dequant w4a16_gemm lora_shrink lora_expand",
+    "comm": ("allreduce_rmsnorm one_shot_ar_rmsnorm ipc_handle ipc_open "
+             "ipc_close"),
+    "mix": ("causal_conv_update gated_delta_rule rglru_scan "
+            "qk_norm_cache_write window_attention post_norm_residual "
+            "rms_norm_cast"),
+}.items():
+    for _n in _names.split():
+        _OP_GROUP[_n] = _g
+
+# groups that predate the split: load_extension() without arguments loads
+# these, so `ops.load_extension(); torch.ops.kaito.<op>` keeps working
+_LEGACY_GROUPS = ("core", "attn", "mla", "moe", "quant", "comm")
 
 
-def extension_available() -> bool:
-    return SO_PATH.exists()
+def extension_available(group: str = "core") -> bool:
+    return so_path(group).exists()
 
 
-def load_extension() -> None:
-    """Load (and lazily build) the HIP extension library."""
-    global _LOADED
-    if _LOADED:
-        return
-    if not SO_PATH.exists():
-        from ._build import build
-        build()
-    torch.ops.load_library(str(SO_PATH))
-    _LOADED = True
+def load_extension(*groups: str) -> None:
+    """Load (and build, if absent) kernel groups; no arguments = every
+    group except the lazily-loaded newer ones."""
+    for g in (groups or _LEGACY_GROUPS):
+        if g in _LOADED:
+            continue
+        if not so_path(g).exists():
+            from ._build import build
+            build(groups=[g])
+        torch.ops.load_library(str(so_path(g)))
+        _LOADED.add(g)
+
+
+class _Kernels:
+    """`_K.<op>` = torch.ops.kaito.<op> with its group loaded first."""
+
+    def __getattr__(self, name: str):
+        group = _OP_GROUP[name]
+        if group not in _LOADED:
+            if not torch.cuda.is_available():
+                raise RuntimeError(
+                    "kaito_amd.ops: got a CUDA tensor but torch.cuda is "
+                    "unavailable")
+            load_extension(group)
+        fn = getattr(torch.ops.kaito, name)
+        setattr(self, name, fn)
+        return fn
+
+
+_K = _Kernels()
 
 
 def _require_ext() -> None:
-    if not _LOADED:
-        if not torch.cuda.is_available():
-            raise RuntimeError(
-                "kaito_amd.ops: got a CUDA tensor but torch.cuda is unavailable")
-        load_extension()
+    """Kept for callers that predate per-group loading (no-op: `_K`
+    loads the group an op needs)."""
 
 
 # ---------------------------------------------------------------- public ops
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     if x.is_cuda:
-        _require_ext()
         out = torch.empty_like(x)
-        torch.ops.kaito.rms_norm(out, x, weight, eps)
+        _K.rms_norm(out, x, weight, eps)
         return out
     return torch_ref.rms_norm(x, weight, eps)
 
@@ -56,9 +100,8 @@ def fused_add_rms_norm(x: torch.Tensor, residual: torch.Tensor,
     """Returns (normed, residual). On GPU, `residual` is updated IN PLACE
     (residual += x) and returned."""
     if x.is_cuda:
-        _require_ext()
         out = torch.empty_like(x)
-        torch.ops.kaito.fused_add_rms_norm(out, x, residual, weight, eps)
+        _K.fused_add_rms_norm(out, x, residual, weight, eps)
         return out, residual
     return torch_ref.fused_add_rms_norm(x, residual, weight, eps)
 
@@ -67,18 +110,20 @@ def rotary_embedding(positions: torch.Tensor, q: torch.Tensor, k: torch.Tensor,
                      head_dim: int, cos_sin_cache: torch.Tensor):
     """In-place on GPU; returns (q, k)."""
     if q.is_cuda:
-        _require_ext()
-        torch.ops.kaito.rotary_embedding(positions, q, k, head_dim, cos_sin_cache)
+        _K.rotary_embedding(positions, q, k, head_dim, cos_sin_cache)
         return q, k
     return torch_ref.rotary_embedding(positions, q, k, head_dim, cos_sin_cache)
 
 
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    if x.is_cuda and x.dtype == torch.float32:
+        # f32 verification mode: plain elementwise math, no bf16 kernel
+        d = x.size(-1) // 2
+        return torch.nn.functional.silu(x[..., :d]) * x[..., d:]
     if x.is_cuda:
-        _require_ext()
         d = x.size(-1) // 2
         out = torch.empty(*x.shape[:-1], d, dtype=x.dtype, device=x.device)
-        torch.ops.kaito.silu_and_mul(out, x)
+        _K.silu_and_mul(out, x)
         return out
     return torch_ref.silu_and_mul(x)
 
@@ -87,8 +132,7 @@ def reshape_and_cache(k: torch.Tensor, v: torch.Tensor, k_cache: torch.Tensor,
                       v_cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
     """k/v: [T, KH, D] (rows may be strided views into a fused qkv buffer)."""
     if k.is_cuda:
-        _require_ext()
-        torch.ops.kaito.reshape_and_cache(k, v, k_cache, v_cache, slot_mapping)
+        _K.reshape_and_cache(k, v, k_cache, v_cache, slot_mapping)
         return
     torch_ref.reshape_and_cache(k, v, k_cache, v_cache, slot_mapping)
 
@@ -114,16 +158,15 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     scale: float, window: int = 0,
                     sinks: torch.Tensor | None = None) -> torch.Tensor:
     if q.is_cuda:
-        _require_ext()
         out = torch.empty_like(q)
         if _PA_IMPL == "sp" or window > 0 or sinks is not None \
                 or k_cache.dtype == torch.uint8:
             # window/sink support lives in the split-phase kernel only
-            torch.ops.kaito.paged_attention_sp(
+            _K.paged_attention_sp(
                 out, q, k_cache, v_cache, block_tables, seq_lens, scale,
                 window, _sinks_arg(sinks, q.device))
         else:
-            torch.ops.kaito.paged_attention(out, q, k_cache, v_cache,
+            _K.paged_attention(out, q, k_cache, v_cache,
                                             block_tables, seq_lens, scale)
         return out
     return torch_ref.paged_attention(q, k_cache, v_cache, block_tables,
@@ -136,10 +179,9 @@ def mla_decode(q: torch.Tensor, cache: torch.Tensor,
     """Absorbed MLA decode over the compressed latent cache (DeepSeek).
     q: [T, H, r+rope]; cache: [NB, BS, r+rope] bf16. Returns [T, H, r]."""
     if q.is_cuda:
-        _require_ext()
         out = torch.empty(q.size(0), q.size(1), r, dtype=q.dtype,
                           device=q.device)
-        torch.ops.kaito.mla_decode(out, q, cache, block_tables, seq_lens,
+        _K.mla_decode(out, q, cache, block_tables, seq_lens,
                                    scale)
         return out
     return torch_ref.mla_decode(q, cache, block_tables, seq_lens, scale, r)
@@ -149,8 +191,7 @@ def mla_cache_write(cache: torch.Tensor, c_kv: torch.Tensor,
                     k_pe: torch.Tensor, slots: torch.Tensor) -> None:
     """Scatter latent rows (c_kv ‖ k_pe) into the paged MLA cache;
     negative slots (graph-bucket padding) are skipped."""
-    _require_ext()
-    torch.ops.kaito.mla_cache_write(cache, c_kv, k_pe, slots)
+    _K.mla_cache_write(cache, c_kv, k_pe, slots)
 
 
 def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
@@ -158,10 +199,9 @@ def prefill_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                       max_seqlen: int | None = None, window: int = 0,
                       sinks: torch.Tensor | None = None) -> torch.Tensor:
     if q.is_cuda:
-        _require_ext()
         out = torch.empty_like(q)
         tile_seq, tile_qbase = _build_tiles(cu_seqlens)
-        torch.ops.kaito.prefill_attention(out, q, k, v, tile_seq, tile_qbase,
+        _K.prefill_attention(out, q, k, v, tile_seq, tile_qbase,
                                           cu_seqlens, scale, window,
                                           _sinks_arg(sinks, q.device))
         return out
@@ -177,10 +217,9 @@ def context_attention(q: torch.Tensor, k_cache: torch.Tensor,
     """Suffix-query causal attention over the paged cache (chunked
     prefill / prefix-cache continuation)."""
     if q.is_cuda:
-        _require_ext()
         out = torch.empty_like(q)
         tile_seq, tile_qbase = _build_tiles(cu_seqlens_q)
-        torch.ops.kaito.context_attention(out, q, k_cache, v_cache, tile_seq,
+        _K.context_attention(out, q, k_cache, v_cache, tile_seq,
                                           tile_qbase, cu_seqlens_q, kv_lens,
                                           block_tables, scale, window,
                                           _sinks_arg(sinks, q.device))
@@ -193,10 +232,9 @@ def context_attention(q: torch.Tensor, k_cache: torch.Tensor,
 def gelu_and_mul(x: torch.Tensor) -> torch.Tensor:
     """GeGLU: gelu_tanh(x[..., :d]) * x[..., d:] (gemma MLPs)."""
     if x.is_cuda:
-        _require_ext()
         d = x.size(-1) // 2
         out = torch.empty(*x.shape[:-1], d, dtype=x.dtype, device=x.device)
-        torch.ops.kaito.gelu_and_mul(out, x)
+        _K.gelu_and_mul(out, x)
         return out
     return torch_ref.gelu_and_mul(x)
 
@@ -204,9 +242,8 @@ def gelu_and_mul(x: torch.Tensor) -> torch.Tensor:
 def gelu(x: torch.Tensor) -> torch.Tensor:
     """Plain tanh-approx GELU (phi-2 ungated MLP)."""
     if x.is_cuda:
-        _require_ext()
         out = torch.empty_like(x)
-        torch.ops.kaito.gelu(out, x.contiguous())
+        _K.gelu(out, x.contiguous())
         return out
     return torch_ref.gelu_tanh(x)
 
@@ -214,11 +251,10 @@ def gelu(x: torch.Tensor) -> torch.Tensor:
 def layer_norm(x: torch.Tensor, weight: torch.Tensor,
                bias: torch.Tensor | None, eps: float) -> torch.Tensor:
     if x.is_cuda:
-        _require_ext()
         out = torch.empty_like(x)
         b = bias if bias is not None else \
             torch.empty(0, dtype=x.dtype, device=x.device)
-        torch.ops.kaito.layer_norm(out, x, weight, b, eps)
+        _K.layer_norm(out, x, weight, b, eps)
         return out
     return torch_ref.layer_norm(x, weight, bias, eps)
 
@@ -228,19 +264,17 @@ def fused_add_layer_norm(x: torch.Tensor, residual: torch.Tensor,
                          eps: float):
     """Returns (normed, residual); residual += x in place on GPU."""
     if x.is_cuda:
-        _require_ext()
         out = torch.empty_like(x)
         b = bias if bias is not None else \
             torch.empty(0, dtype=x.dtype, device=x.device)
-        torch.ops.kaito.fused_add_layer_norm(out, x, residual, weight, b, eps)
+        _K.fused_add_layer_norm(out, x, residual, weight, b, eps)
         return out, residual
     new_res = (x.float() + residual.float()).to(x.dtype)
     return torch_ref.layer_norm(new_res, weight, bias, eps), new_res
 
 
 def mfma_tile_gemm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    _require_ext()
-    return torch.ops.kaito.mfma_tile_gemm(a, b)
+    return _K.mfma_tile_gemm(a, b)
 
 
 QTILE = 64  # must match prefill_attention.hip
@@ -269,9 +303,8 @@ def moe_gate_silu(act: torch.Tensor, x: torch.Tensor,
     gate/up grouped GEMM per expert, activation epilogue into `act`
     (act_mode 0 = SwiGLU, 1 = gpt-oss clamped swiglu; optional
     per-expert [E, 2*IE] bias)."""
-    _require_ext()
     b = bias if bias is not None else         torch.empty(0, dtype=x.dtype, device=x.device)
-    torch.ops.kaito.moe_gate_silu(act, x, w_gate_up, sorted_ids, offsets,
+    _K.moe_gate_silu(act, x, w_gate_up, sorted_ids, offsets,
                                   b, act_mode, e_base, n_local_experts)
 
 
@@ -282,9 +315,8 @@ def moe_down_scatter(out: torch.Tensor, act: torch.Tensor,
                      bias: torch.Tensor | None = None) -> None:
     """Fused MoE stage 2 (GPU only): down grouped GEMM (+ optional
     [E, H] bias) + gated f32 atomic scatter into `out`."""
-    _require_ext()
     b = bias if bias is not None else         torch.empty(0, dtype=act.dtype, device=act.device)
-    torch.ops.kaito.moe_down_scatter(out, act, w_down, sorted_ids, gates,
+    _K.moe_down_scatter(out, act, w_down, sorted_ids, gates,
                                      offsets, b, e_base, n_local_experts)
 
 
@@ -293,10 +325,9 @@ def w4a16_gemv(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     """Group-quantized W4A16 linear, small M (decode): out = x @ W^T with
     W dequantized on the fly inside the kernel."""
     if x.is_cuda:
-        _require_ext()
         out = torch.empty(x.size(0), qweight.size(0), dtype=x.dtype,
                           device=x.device)
-        torch.ops.kaito.w4a16_gemv(out, x, qweight, scales, zeros, group)
+        _K.w4a16_gemv(out, x, qweight, scales, zeros, group)
         return out
     return torch_ref.w4a16_gemv(x, qweight, scales, zeros, group)
 
@@ -307,11 +338,10 @@ def w4a16_dequant(qweight: torch.Tensor, scales: torch.Tensor,
     """Dequantize packed 4-bit weights to bf16 [N, K] (feeds hipBLASLt
     MFMA for large-M GEMMs)."""
     if qweight.is_cuda:
-        _require_ext()
         if out is None:
             out = torch.empty(qweight.size(0), qweight.size(1) * 8,
                               dtype=torch.bfloat16, device=qweight.device)
-        torch.ops.kaito.w4a16_dequant(out, qweight, scales, zeros, group)
+        _K.w4a16_dequant(out, qweight, scales, zeros, group)
         return out
     ref = torch_ref.w4a16_unpack(qweight, scales, zeros, group)
     return ref.to(torch.bfloat16) if out is None else out.copy_(ref)
@@ -323,10 +353,133 @@ def w4a16_gemm(x: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
     The 4-bit weights never round-trip through a full-precision scratch
     buffer. CPU falls back to the unpack reference."""
     if x.is_cuda:
-        _require_ext()
         out = torch.empty(x.size(0), qweight.size(0), dtype=x.dtype,
                           device=x.device)
-        torch.ops.kaito.w4a16_gemm(out, x.contiguous(), qweight, scales,
+        _K.w4a16_gemm(out, x.contiguous(), qweight, scales,
                                    zeros, group)
         return out
     return torch_ref.w4a16_gemv(x, qweight, scales, zeros, group)
+
+
+# ---- stateful sequence mixers (hybrid stacks; kernel group "mix") --------
+#
+# Batch layout shared by these ops: the rows of all chunks of a step are
+# concatenated; chunk b owns rows cu_seqlens[b]..cu_seqlens[b+1], belongs
+# to the sequence held in state slot state_slots[b] (<0: padding, skipped)
+# and starts at sequence position seq_starts[b] (0: fresh sequence, the
+# slot's old content is ignored). token_seq[t] is the chunk of row t.
+# Activations may be bf16 or f32 (one dtype per call); states, small
+# per-channel parameters and all recurrence math are f32.
+
+def _none(t, like):
+    return t if t is not None else \
+        torch.empty(0, dtype=torch.float32, device=like.device)
+
+
+def causal_conv_update(x, weight, bias, conv_state, cu_seqlens, state_slots,
+                       seq_starts, token_seq, act: int = 0):
+    """Depthwise causal short convolution with a carried tail.
+    x [T, C] (row stride free); weight [C, taps] f32; conv_state
+    [slots, taps-1, C] in x's dtype, advanced in place; act 0 none,
+    1 silu. Returns [T, C]."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _K.causal_conv_update(out, x, weight, _none(bias, x), conv_state,
+                              cu_seqlens, state_slots, seq_starts, token_seq,
+                              act)
+        return out
+    return torch_ref.causal_conv_update(x, weight, bias, conv_state,
+                                        cu_seqlens, state_slots, seq_starts,
+                                        act)
+
+
+def gated_delta_rule(q, k, v, gate, a, b, a_log, dt_bias, norm_w, state,
+                     cu_seqlens, state_slots, seq_starts, qk_eps: float,
+                     norm_eps: float):
+    """Gated delta rule with fused unit-norm of q/k, decay/beta
+    activations, output RMS norm and silu gate. q/k [T, G, D], v/gate
+    [T, H, V], a/b [T, H] (row strides free); state [slots, H, D, V] f32
+    in place. Returns [T, H*V]."""
+    if v.is_cuda:
+        T, H, V = v.shape
+        out = torch.empty(T, H * V, dtype=v.dtype, device=v.device)
+        _K.gated_delta_rule(out, q, k, v, gate, a, b, a_log, dt_bias, norm_w,
+                            state, cu_seqlens, state_slots, seq_starts,
+                            qk_eps, norm_eps)
+        return out
+    return torch_ref.gated_delta_rule(
+        q, k, v, gate, a, b, a_log, dt_bias, norm_w, state, cu_seqlens,
+        state_slots, seq_starts, qk_eps, norm_eps).reshape(v.size(0), -1)
+
+
+def rglru_scan(u, gates, y, decay_rate, state, cu_seqlens, state_slots,
+               seq_starts):
+    """Real-gated linear recurrence + GELU gate branch. u/y [T, W] (row
+    strides free); gates [B, T, 2*W/B] f32; decay_rate [W] f32; state
+    [slots, W] f32 in place. Returns [T, W]."""
+    if u.is_cuda:
+        out = torch.empty(u.shape, dtype=u.dtype, device=u.device)
+        _K.rglru_scan(out, u, gates, y, decay_rate, state, cu_seqlens,
+                      state_slots, seq_starts)
+        return out
+    return torch_ref.rglru_scan(u, gates, y, decay_rate, state, cu_seqlens,
+                                state_slots, seq_starts)
+
+
+def qk_norm_cache_write(q, k, v, q_w, k_w, eps: float, k_cache, v_cache,
+                        slot_mapping):
+    """Per-head RMS norm of q [T, H, D] / k [T, G, D] (f32 weights [D] or
+    None) fused with the scatter of k and v [T, G, V] into the paged
+    caches [blocks, G, block_size, D|V]. Returns normed q [T, H, D]."""
+    if q.is_cuda:
+        qn = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        _K.qk_norm_cache_write(qn, q, k, v, _none(q_w, q), _none(k_w, q),
+                               eps, k_cache, v_cache, slot_mapping)
+        return qn
+    return torch_ref.qk_norm_cache_write(q, k, v, q_w, k_w, eps, k_cache,
+                                         v_cache, slot_mapping)
+
+
+def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
+                     scale: float, softcap: float = 0.0, r1=None, r2=None,
+                     window: int = 0):
+    """Causal sliding-window attention of query rows [T, H, D] over the
+    paged cache (key size D, value size V may differ), with optional tanh
+    score capping and the distance penalty r1*ln(1 + r2*distance).
+    Returns [T, H, V]."""
+    if q.is_cuda:
+        T, H, _ = q.shape
+        out = torch.empty(T, H, v_cache.size(3), dtype=q.dtype,
+                          device=q.device)
+        _K.window_attention(out, q, k_cache, v_cache, block_tables, token_seq,
+                            positions, scale, softcap, _none(r1, q),
+                            _none(r2, q), window)
+        return out
+    return torch_ref.window_attention(q, k_cache, v_cache, block_tables,
+                                      token_seq, positions, scale, softcap,
+                                      r1, r2, window)
+
+
+def post_norm_residual(x32, y, w, eps: float, out_dtype, y2=None, w_y=None,
+                       w_y2=None):
+    """x32 [T, H] f32 += rms(m) * w in place, m = y or, with y2,
+    (rms(y)*w_y + rms(y2)*w_y2)/2. Returns x32 rounded to out_dtype."""
+    if x32.is_cuda:
+        if out_dtype == torch.float32:
+            xo = x32
+        else:
+            xo = torch.empty(x32.shape, dtype=out_dtype, device=x32.device)
+        _K.post_norm_residual(x32, xo, y, w, eps, _none(y2, y),
+                              _none(w_y, y), _none(w_y2, y))
+        return xo
+    return torch_ref.post_norm_residual(x32, y, w, eps, out_dtype, y2, w_y,
+                                        w_y2)
+
+
+def rms_norm_cast(x, weight, eps: float, out_dtype):
+    """RMS norm of f32 or bf16 rows with an f32 weight → out_dtype."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _K.rms_norm_cast(out, x, weight, eps)
+        return out
+    return torch_ref.rms_norm_cast(x, weight, eps, out_dtype)

@@ -1,0 +1,311 @@
+// Softmax attention over a sliding window of the paged K/V cache with a
+// distance penalty, for batches of chunks (prompt portions and single
+// decode tokens alike), plus the fused per-head qk RMS norm + cache write.
+//
+//   score(i, j) = cap * tanh(q_i . k_j * scale / cap)      (cap > 0)
+//                 - r1_h * ln(1 + r2_h * (i - j))           (r1 given)
+//   visible:      0 <= i - j < window   (window <= 0: every j <= i)
+//
+// Key size D and value size V are independent; caches are
+// [blocks, G, block_size, D|V] in the activation dtype. Scores, softmax
+// weights and the output accumulation are f32.
+//
+// window_attention_kernel: one workgroup per (query row, head). Keys are
+// taken a tile of blockDim keys at a time: one thread scores one key
+// (vector loads of its cache row), the tile's weights go through LDS, and
+// the P·V product is thread-per-value-dim, so consecutive lanes read
+// consecutive cache elements. Tiles are folded with the running-max
+// (online softmax) recurrence, so any window length works.
+#include "mix_common.h"
+
+namespace kaito {
+
+namespace {
+
+// ---- q/k norm + cache scatter -------------------------------------------
+// grid (T, H + 2G): blockIdx.y < H → q head; < H+G → k head; else v head.
+template <typename T>
+__global__ void qk_norm_cache_write_kernel(
+    T* __restrict__ q_out,                                   // [T, H, D]
+    const T* __restrict__ q, const int64_t q_s0, const int64_t q_s1,
+    const T* __restrict__ k, const int64_t k_s0, const int64_t k_s1,
+    const T* __restrict__ v, const int64_t v_s0, const int64_t v_s1,
+    const float* __restrict__ q_w, const float* __restrict__ k_w,
+    const float eps, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int64_t* __restrict__ slots, const int H, const int G, const int D,
+    const int V, const int BS) {
+  const int t = blockIdx.x, y = blockIdx.y, lane = threadIdx.x;
+  if (y < H) {
+    const T* src = q + (int64_t)t * q_s0 + (int64_t)y * q_s1;
+    T* dst = q_out + ((int64_t)t * H + y) * D;
+    float inv = 1.0f;
+    if (q_w != nullptr) {
+      float ss = 0.f;
+      for (int d = lane; d < D; d += 64) { const float x = act_ld(src + d); ss += x * x; }
+      ss = wave_reduce_sum(ss);
+      inv = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    for (int d = lane; d < D; d += 64)
+      act_st(dst + d, act_ld(src + d) * inv * (q_w ? q_w[d] : 1.0f));
+    return;
+  }
+  const int64_t slot = slots[t];
+  if (slot < 0) return;
+  const int64_t blk = slot / BS;
+  const int off = (int)(slot % BS);
+  if (y < H + G) {
+    const int g = y - H;
+    const T* src = k + (int64_t)t * k_s0 + (int64_t)g * k_s1;
+    T* dst = k_cache + ((blk * G + g) * BS + off) * D;
+    float inv = 1.0f;
+    if (k_w != nullptr) {
+      float ss = 0.f;
+      for (int d = lane; d < D; d += 64) { const float x = act_ld(src + d); ss += x * x; }
+      ss = wave_reduce_sum(ss);
+      inv = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    for (int d = lane; d < D; d += 64)
+      act_st(dst + d, act_ld(src + d) * inv * (k_w ? k_w[d] : 1.0f));
+  } else {
+    const int g = y - H - G;
+    const T* src = v + (int64_t)t * v_s0 + (int64_t)g * v_s1;
+    T* dst = v_cache + ((blk * G + g) * BS + off) * V;
+    for (int d = lane; d < V; d += 64) dst[d] = src[d];
+  }
+}
+
+// ---- attention ------------------------------------------------------------
+template <typename T>
+KAITO_DEV float dot_row(const float* __restrict__ q, const T* __restrict__ k,
+                        const int D);
+
+template <>
+KAITO_DEV float dot_row<float>(const float* __restrict__ q,
+                               const float* __restrict__ k, const int D) {
+  float acc = 0.f;
+  int d = 0;
+  if ((((uintptr_t)k) & 15) == 0) {
+    for (; d + 4 <= D; d += 4) {
+      const float4_t kv = *reinterpret_cast<const float4_t*>(k + d);
+      acc += q[d] * kv[0] + q[d + 1] * kv[1] + q[d + 2] * kv[2] +
+             q[d + 3] * kv[3];
+    }
+  }
+  for (; d < D; d++) acc += q[d] * k[d];
+  return acc;
+}
+
+template <>
+KAITO_DEV float dot_row<bf16_act>(const float* __restrict__ q,
+                                  const bf16_act* __restrict__ k,
+                                  const int D) {
+  float acc = 0.f;
+  int d = 0;
+  if ((((uintptr_t)k) & 15) == 0) {
+    for (; d + 8 <= D; d += 8) {
+      const short8_t kv = *reinterpret_cast<const short8_t*>(k + d);
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc += q[d + i] * bf16_to_f32(kv[i]);
+    }
+  }
+  for (; d < D; d++) acc += q[d] * bf16_to_f32(k[d].v);
+  return acc;
+}
+
+template <typename T>
+__global__ void window_attention_kernel(
+    T* __restrict__ out,                                   // [T, H, V]
+    const T* __restrict__ q,                               // [T, H, D]
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_tables, const int max_blocks,
+    const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
+    const float scale, const float softcap, const float* __restrict__ r1,
+    const float* __restrict__ r2, const int window, const int H, const int G,
+    const int D, const int V, const int BS) {
+  extern __shared__ float lds[];
+  const int KT = blockDim.x;            // keys per tile
+  float* q_s = lds;                     // [D]
+  float* p_s = lds + D;                 // [KT]
+  int* blk_s = reinterpret_cast<int*>(p_s + KT);   // [KT] cache row bases
+  __shared__ float red[16];
+  __shared__ float bcast[2];
+
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int b = token_seq[t];
+  T* orow = out + ((int64_t)t * H + h) * V;
+  if (b < 0) {
+    for (int j = tid; j < V; j += KT) act_st(orow + j, 0.0f);
+    return;
+  }
+  const int g = h / (H / G);
+  const int pos = (int)positions[t];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int nkeys = pos - lo + 1;
+  const int* bt = block_tables + (int64_t)b * max_blocks;
+  const float hr1 = r1 ? r1[h] : 0.0f, hr2 = r1 ? r2[h] : 0.0f;
+
+  for (int d = tid; d < D; d += KT)
+    q_s[d] = act_ld(q + ((int64_t)t * H + h) * D + d);
+
+  // output dims owned by this thread: j = tid + i*KT
+  constexpr int MAXV = 4;               // V <= 4 * blockDim
+  float acc[MAXV];
+#pragma unroll
+  for (int i = 0; i < MAXV; i++) acc[i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  for (int k0 = 0; k0 < nkeys; k0 += KT) {
+    const int nk = min(KT, nkeys - k0);
+    __syncthreads();                    // q_s ready / previous tile consumed
+    float s = -INFINITY;
+    if (tid < nk) {
+      const int j = lo + k0 + tid;
+      const int page = bt[j / BS];
+      const int64_t rowi = ((int64_t)page * G + g) * BS + (j % BS);
+      blk_s[tid] = (int)rowi;
+      s = dot_row<T>(q_s, k_cache + rowi * D, D) * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      if (r1) s -= hr1 * log1pf(hr2 * (float)(pos - j));
+    }
+    // tile max
+    float mx = wave_reduce_max(s);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    if (tid == 0) {
+      float m = red[0];
+      for (int w = 1; w < (KT >> 6); w++) m = fmaxf(m, red[w]);
+      bcast[0] = m;
+    }
+    __syncthreads();
+    const float m_new = fmaxf(m_run, bcast[0]);
+    const float p = tid < nk ? expf(s - m_new) : 0.f;
+    p_s[tid] = p;
+    float ps = wave_reduce_sum(p);
+    __syncthreads();                    // red[] free again; p_s visible
+    if ((tid & 63) == 0) red[tid >> 6] = ps;
+    __syncthreads();
+    float tile_sum = 0.f;
+    for (int w = 0; w < (KT >> 6); w++) tile_sum += red[w];
+    const float corr = expf(m_run - m_new);     // 0 on the first tile
+    l_run = l_run * corr + tile_sum;
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < MAXV; i++) {
+      const int j = tid + i * KT;
+      if (j < V) {
+        float a = acc[i] * corr;
+        for (int kk = 0; kk < nk; kk++)
+          a += p_s[kk] * act_ld(v_cache + (int64_t)blk_s[kk] * V + j);
+        acc[i] = a;
+      }
+    }
+  }
+  const float inv = 1.0f / l_run;
+#pragma unroll
+  for (int i = 0; i < MAXV; i++) {
+    const int j = tid + i * KT;
+    if (j < V) act_st(orow + j, acc[i] * inv);
+  }
+}
+
+}  // namespace
+
+void qk_norm_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor k,
+                         at::Tensor v, at::Tensor q_w, at::Tensor k_w,
+                         double eps, at::Tensor k_cache, at::Tensor v_cache,
+                         at::Tensor slot_mapping) {
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && k.dim() == 3 && v.dim() == 3);
+  const int T = q.size(0), H = q.size(1), D = q.size(2);
+  const int G = k.size(1), V = v.size(2);
+  TORCH_CHECK(k.size(0) == T && v.size(0) == T && k.size(2) == D &&
+              v.size(1) == G);
+  for (const at::Tensor* t : {&q, &k, &v})
+    TORCH_CHECK(t->stride(2) == 1 && t->dtype() == q.dtype());
+  TORCH_CHECK(is_act_dtype(q) && q_out.is_contiguous() &&
+              q_out.sizes() == q.sizes() && q_out.dtype() == q.dtype());
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.dtype() == q.dtype() && v_cache.dtype() == q.dtype());
+  TORCH_CHECK(k_cache.size(1) == G && k_cache.size(3) == D &&
+              v_cache.size(1) == G && v_cache.size(3) == V &&
+              v_cache.size(0) == k_cache.size(0) &&
+              v_cache.size(2) == k_cache.size(2));
+  const int BS = k_cache.size(2);
+  const bool qn = q_w.numel() > 0, kn = k_w.numel() > 0;
+  if (qn) { KAITO_CHECK_F32(q_w); TORCH_CHECK(q_w.numel() == D); }
+  if (kn) { KAITO_CHECK_F32(k_w); TORCH_CHECK(k_w.numel() == D); }
+  TORCH_CHECK(slot_mapping.is_cuda() && slot_mapping.dtype() == at::kLong &&
+              slot_mapping.is_contiguous() && slot_mapping.size(0) == T);
+  if (T == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+  KAITO_DISPATCH_ACT(q, {
+    hipLaunchKernelGGL((qk_norm_cache_write_kernel<act_t>),
+        dim3(T, H + 2 * G), dim3(64), 0, stream, (act_t*)q_out.data_ptr(),
+        (const act_t*)q.data_ptr(), q.stride(0), q.stride(1),
+        (const act_t*)k.data_ptr(), k.stride(0), k.stride(1),
+        (const act_t*)v.data_ptr(), v.stride(0), v.stride(1),
+        qn ? q_w.data_ptr<float>() : nullptr,
+        kn ? k_w.data_ptr<float>() : nullptr, (float)eps,
+        (act_t*)k_cache.data_ptr(), (act_t*)v_cache.data_ptr(),
+        slot_mapping.data_ptr<int64_t>(), H, G, D, V, BS);
+  });
+}
+
+void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
+                      at::Tensor v_cache, at::Tensor block_tables,
+                      at::Tensor token_seq, at::Tensor positions,
+                      double scale, double softcap, at::Tensor r1,
+                      at::Tensor r2, int64_t window) {
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() &&
+              is_act_dtype(q));
+  const int T = q.size(0), H = q.size(1), D = q.size(2);
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.dtype() == q.dtype() && v_cache.dtype() == q.dtype());
+  const int G = k_cache.size(1), BS = k_cache.size(2), V = v_cache.size(3);
+  TORCH_CHECK(k_cache.size(3) == D && v_cache.size(1) == G &&
+              v_cache.size(2) == BS && H % G == 0);
+  TORCH_CHECK(out.is_contiguous() && out.dtype() == q.dtype() &&
+              out.dim() == 3 && out.size(0) == T && out.size(1) == H &&
+              out.size(2) == V);
+  KAITO_CHECK_I32(block_tables); KAITO_CHECK_I32(token_seq);
+  TORCH_CHECK(block_tables.dim() == 2 && token_seq.size(0) == T);
+  TORCH_CHECK(positions.is_cuda() && positions.dtype() == at::kLong &&
+              positions.is_contiguous() && positions.size(0) == T);
+  const bool bias = r1.numel() > 0;
+  if (bias) {
+    KAITO_CHECK_F32(r1); KAITO_CHECK_F32(r2);
+    TORCH_CHECK(r1.numel() == H && r2.numel() == H);
+  }
+  TORCH_CHECK((int64_t)k_cache.size(0) * G * BS < (1ll << 31));
+  if (T == 0) return;
+  // keys per tile: the window when it is short, else 256
+  int threads = 256;
+  if (window > 0 && window <= 64) threads = 64;
+  else if (window > 0 && window <= 128) threads = 128;
+  while (4 * threads < V) threads <<= 1;
+  TORCH_CHECK(threads <= 1024, "value size too large: ", V);
+  const size_t lds_bytes = ((size_t)D + 2 * threads) * 4;
+  auto stream = at::hip::getCurrentHIPStream();
+  KAITO_DISPATCH_ACT(q, {
+    hipLaunchKernelGGL((window_attention_kernel<act_t>), dim3(T, H),
+        dim3(threads), lds_bytes, stream, (act_t*)out.data_ptr(),
+        (const act_t*)q.data_ptr(), (const act_t*)k_cache.data_ptr(),
+        (const act_t*)v_cache.data_ptr(), block_tables.data_ptr<int>(),
+        (int)block_tables.size(1), token_seq.data_ptr<int>(),
+        positions.data_ptr<int64_t>(), (float)scale, (float)softcap,
+        bias ? r1.data_ptr<float>() : nullptr,
+        bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, D, V, BS);
+  });
+}
+
+}  // namespace kaito
+
+TORCH_LIBRARY_FRAGMENT(kaito, m) {
+  m.def("qk_norm_cache_write(Tensor(a!) q_out, Tensor q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, float eps, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slot_mapping) -> ()");
+  m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor token_seq, Tensor positions, float scale, float softcap, Tensor r1, Tensor r2, int window) -> ()");
+}
+TORCH_LIBRARY_IMPL(kaito, CUDA, m) {
+  m.impl("qk_norm_cache_write", &kaito::qk_norm_cache_write);
+  m.impl("window_attention", &kaito::window_attention);
+}

@@ -240,3 +240,184 @@ def mla_decode(q: torch.Tensor, cache: torch.Tensor,
         p = torch.softmax(s, dim=-1)
         out[i] = (p @ rows[:, :r]).to(out.dtype)
     return out
+
+
+# ---- sequence mixers with per-sequence state (hybrid stacks) -------------
+#
+# Shared batch layout: rows of all chunks are concatenated; chunk b owns
+# rows cu[b]..cu[b+1], continues the sequence held in state slot slots[b]
+# and starts at sequence position starts[b] (0 = fresh sequence: the state
+# is taken as zero and the slot's old content is ignored). Slots < 0 mark
+# padding chunks, which are skipped.
+
+def _chunks(cu_seqlens, state_slots, seq_starts):
+    cu = cu_seqlens.tolist()
+    sl = state_slots.tolist()
+    st = seq_starts.tolist()
+    for b in range(len(sl)):
+        if sl[b] >= 0 and cu[b + 1] > cu[b]:
+            yield cu[b], cu[b + 1], sl[b], st[b]
+
+
+def causal_conv_update(x, weight, bias, conv_state, cu_seqlens, state_slots,
+                       seq_starts, act: int):
+    """Depthwise causal convolution over time. x [T, C]; weight [C, taps]
+    (last column multiplies the current token); conv_state
+    [slots, taps-1, C] holds each sequence's last taps-1 inputs and is
+    advanced in place. act: 0 none, 1 silu."""
+    taps = weight.size(1)
+    out = torch.empty_like(x)
+    w = weight.float()
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        prev = conv_state[slot].float() if start > 0 else \
+            torch.zeros(taps - 1, x.size(1))
+        seq = torch.cat([prev, x[r0:r1].float()], 0)
+        n = r1 - r0
+        acc = torch.zeros(n, x.size(1))
+        for j in range(taps):
+            acc += seq[j:j + n] * w[:, j]
+        if bias is not None:
+            acc += bias.float()
+        if act == 1:
+            acc = torch.nn.functional.silu(acc)
+        out[r0:r1] = acc.to(x.dtype)
+        if taps > 1:
+            conv_state[slot] = seq[n:].to(conv_state.dtype)
+    return out
+
+
+def gated_delta_rule(q, k, v, gate, a, b, a_log, dt_bias, norm_w, state,
+                     cu_seqlens, state_slots, seq_starts, qk_eps: float,
+                     norm_eps: float):
+    """q/k [T, G, D], v/gate [T, H, V], a/b [T, H]; state [slots, H, D, V]
+    f32, advanced in place. Per token and head: decay the state, write the
+    beta-scaled prediction error along k, read out along q; the read-out
+    is RMS-normed, weighted and gated by silu(gate)."""
+    T, G, D = q.shape
+    H, V = v.shape[1], v.shape[2]
+    rep = H // G
+    qf, kf, vf = q.float(), k.float(), v.float()
+    qf = qf * torch.rsqrt(qf.pow(2).sum(-1, keepdim=True) + qk_eps) * D ** -0.5
+    kf = kf * torch.rsqrt(kf.pow(2).sum(-1, keepdim=True) + qk_eps)
+    qf = qf.repeat_interleave(rep, 1)
+    kf = kf.repeat_interleave(rep, 1)
+    beta = torch.sigmoid(b.float())
+    decay = torch.exp(-torch.exp(a_log.float()) *
+                      torch.nn.functional.softplus(a.float() + dt_bias.float()))
+    o = torch.zeros(T, H, V)
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        S = state[slot].clone() if start > 0 else torch.zeros(H, D, V)
+        for t in range(r0, r1):
+            S = S * decay[t, :, None, None]
+            pred = torch.einsum("hdv,hd->hv", S, kf[t])
+            u = beta[t, :, None] * (vf[t] - pred)
+            S = S + kf[t, :, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slot] = S
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + norm_eps)
+    o = o * norm_w.float() * torch.nn.functional.silu(gate.float())
+    return o.to(v.dtype)
+
+
+def rglru_scan(u, gates, y, decay_rate, state, cu_seqlens, state_slots,
+               seq_starts):
+    """Real-gated linear recurrent unit. u, y [T, W]; gates [B, T, 2*bw]
+    f32 pre-activations (recurrence gate | input gate per block of
+    bw = W // B channels); decay_rate [W] f32 (already multiplied by the
+    design's constant); state [slots, W] f32, advanced in place.
+    out = S_t * gelu_tanh(y)."""
+    T, W = u.shape
+    B = gates.size(0)
+    bw = W // B
+    g = gates.float().permute(1, 0, 2)                   # [T, B, 2bw]
+    r = torch.sigmoid(g[..., :bw]).reshape(T, W)
+    i = torch.sigmoid(g[..., bw:]).reshape(T, W)
+    log_a = -r * decay_rate.float()
+    a = torch.exp(log_a)
+    drive = torch.sqrt(1.0 - a * a) * i * u.float()
+    out = torch.empty(T, W)
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        S = state[slot].clone() if start > 0 else torch.zeros(W)
+        for t in range(r0, r1):
+            S = a[t] * S + drive[t]
+            out[t] = S
+        state[slot] = S
+    return (out * gelu_tanh(y.float())).to(u.dtype)
+
+
+def qk_norm_cache_write(q, k, v, q_w, k_w, eps: float, k_cache, v_cache,
+                        slot_mapping):
+    """Per-head RMS norm of q [T, H, D] and k [T, G, D] (weights [D], or
+    None for no norm), then scatter k and v [T, G, V] into the paged
+    caches [blocks, G, block_size, D|V]. Returns the normed q."""
+    def norm(t, w):
+        if w is None:
+            return t
+        tf = t.float()
+        return (tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps)
+                * w.float()).to(t.dtype)
+    qn, kn = norm(q, q_w), norm(k, k_w)
+    bs = k_cache.size(2)
+    for t, slot in enumerate(slot_mapping.tolist()):
+        if slot < 0:
+            continue
+        k_cache[slot // bs, :, slot % bs] = kn[t].to(k_cache.dtype)
+        v_cache[slot // bs, :, slot % bs] = v[t].to(v_cache.dtype)
+    return qn
+
+
+def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
+                     scale: float, softcap: float, r1, r2, window: int):
+    """Causal sliding-window attention of query rows over the paged cache.
+    Row t belongs to chunk token_seq[t] (its block table row) at sequence
+    position positions[t] and sees keys j with 0 <= pos - j < window
+    (window <= 0: all earlier keys). score = cap(q.k * scale) -
+    r1 * ln(1 + r2 * (pos - j))."""
+    T, H, D = q.shape
+    G, bs, V = k_cache.size(1), k_cache.size(2), v_cache.size(3)
+    rep = H // G
+    out = torch.zeros(T, H, V)
+    pos_l, seq_l = positions.tolist(), token_seq.tolist()
+    for t in range(T):
+        if seq_l[t] < 0:
+            continue
+        p = pos_l[t]
+        lo = max(0, p - window + 1) if window > 0 else 0
+        js = torch.arange(lo, p + 1)
+        blk = block_tables[seq_l[t]].long()[js // bs]
+        kk = k_cache[blk, :, js % bs].float()            # [n, G, D]
+        vv = v_cache[blk, :, js % bs].float()
+        kk = kk.repeat_interleave(rep, 1)
+        vv = vv.repeat_interleave(rep, 1)
+        s = torch.einsum("hd,nhd->hn", q[t].float(), kk) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        if r1 is not None:
+            dist = (p - js).float()
+            s = s - r1.float()[:, None] * torch.log1p(
+                r2.float()[:, None] * dist[None, :])
+        out[t] = torch.einsum("hn,nhv->hv", torch.softmax(s, -1), vv)
+    return out.to(q.dtype)
+
+
+def post_norm_residual(x32, y, w, eps: float, out_dtype, y2=None, w_y=None,
+                       w_y2=None):
+    """Residual update with the norm on the sub-layer OUTPUT:
+    x32 += rms(m) * w, in place, where m = y, or with y2 given
+    m = (rms(y) * w_y + rms(y2) * w_y2) / 2. Returns x32 rounded to
+    out_dtype (the next sub-layer's input)."""
+    def rms(t):
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)
+    m = y.float()
+    if y2 is not None:
+        m = 0.5 * (rms(m) * w_y.float() + rms(y2.float()) * w_y2.float())
+    x32 += rms(m) * w.float()
+    return x32.to(out_dtype)
+
+
+def rms_norm_cast(x, weight, eps: float, out_dtype):
+    """RMS norm of rows of any float dtype with an f32 weight, rounded to
+    out_dtype."""
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+            * weight.float()).to(out_dtype)

@@ -52,7 +52,7 @@ def fused_local(inputs: List[torch.Tensor], weight: torch.Tensor,
         var = acc.pow(2).mean(-1, keepdim=True)
         return (acc * torch.rsqrt(var + eps) *
                 weight.float()).to(inputs[0].dtype)
-    ops.load_extension()
+    ops.load_extension("comm")
     out = torch.empty_like(inputs[0])
     ptrs = torch.tensor([t.data_ptr() for t in inputs], dtype=torch.long,
                         device=inputs[0].device)
@@ -77,7 +77,7 @@ class OneShotGroup:
         self.group = st.tp_group
         self.max_tokens = max_tokens
         self.hidden = hidden
-        ops.load_extension()
+        ops.load_extension("comm")
         # double-buffered staging in ONE allocation (one IPC handle)
         self.buf = torch.empty(2, max_tokens, hidden, dtype=dtype,
                                device="cuda")

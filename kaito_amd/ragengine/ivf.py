@@ -156,7 +156,7 @@ class IVFFlatIndex:
         the query vector up and (nprobe + top_k) scalars down."""
         import torch
         from .. import ops
-        ops.load_extension()
+        ops.load_extension("core")
         vecs, cent, order, offsets = self._gpu_state()
         dev = vecs.device
         q = torch.from_numpy(

@@ -108,7 +108,7 @@ class FlatIndex:
             k = min(top_k, 32)
             vals = torch.empty(1, k, dtype=torch.float32, device="cuda")
             idx = torch.empty(1, k, dtype=torch.int32, device="cuda")
-            ops.load_extension()
+            ops.load_extension("core")
             import torch as _t
             _t.ops.kaito.topk(vals, idx, scores, k)
             vi = idx[0].cpu().tolist()
