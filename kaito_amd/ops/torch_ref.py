@@ -269,7 +269,7 @@ def causal_conv_update(x, weight, bias, conv_state, cu_seqlens, state_slots,
     out = torch.empty_like(x)
     w = weight.float()
     for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
-        prev = conv_state[slot].float() if start > 0 else \
+        prev = conv_state[slot, :taps - 1].float() if start > 0 else \
             torch.zeros(taps - 1, x.size(1))
         seq = torch.cat([prev, x[r0:r1].float()], 0)
         n = r1 - r0
@@ -282,7 +282,7 @@ def causal_conv_update(x, weight, bias, conv_state, cu_seqlens, state_slots,
             acc = torch.nn.functional.silu(acc)
         out[r0:r1] = acc.to(x.dtype)
         if taps > 1:
-            conv_state[slot] = seq[n:].to(conv_state.dtype)
+            conv_state[slot, :taps - 1] = seq[n:].to(conv_state.dtype)
     return out
 
 
