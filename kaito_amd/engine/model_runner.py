@@ -26,7 +26,6 @@ from .scheduler import ScheduledBatch
 from .sequence import Sequence
 from . import lora as lora_mod
 from ..models.llama import AttnMetadata
-from ..models.registry import resolve_model_class
 from ..parallel import state as ps
 
 logger = logging.getLogger(__name__)
@@ -38,6 +37,7 @@ class ModelRunner:
         self.device = torch.device(cfg.device)
         self.is_gpu = self.device.type == "cuda"
         torch.manual_seed(cfg.seed)
+        from ..models.registry import resolve_model_class
         self.model = resolve_model_class(cfg.model)(cfg.model).to(self.device)
         # models whose mixers carry per-sequence recurrent state: the
         # runner sizes a slot per live sequence and always hands the

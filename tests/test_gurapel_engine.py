@@ -1,0 +1,233 @@
+"""The hybrid (Gurapel) model served by the engine against the plain oracle
+in tests/hybrid_oracle.py: whole prompts, token-by-token decoding, portions
+down to two tokens, unequal batches, reuse of pages and state slots, window
+and page borders, far-away tokens, other sizes, greedy generation through
+the scheduler. CPU runs use the engine's reference ops; the same tests run
+on the HIP kernels under `-m gpu` (f32 and bf16)."""
+import random
+
+import pytest
+import torch
+
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import hybrid_oracle as O  # noqa: E402
+
+DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
+MODES = [("cpu", "float32"),
+         pytest.param(("cuda", "float32"), marks=pytest.mark.gpu),
+         pytest.param(("cuda", "bfloat16"), marks=pytest.mark.gpu)]
+
+
+def config_a():
+    # page size is 16: window 11 slides inside and across pages, window 21
+    # always spans two or three
+    return O.make_config([
+        O.delta_layer(heads=2, kv_heads=1, dim=16, vdim=24, conv=3,
+                      mlp=O.moe(4, 2, 24)),
+        O.parallel_layer(heads=4, kv_heads=2, dim=16, vdim=8, window=11,
+                         width=48, blocks=3, conv=2, mlp=O.moe(3, 1, 40)),
+        O.parallel_layer(heads=2, kv_heads=2, dim=8, vdim=24, window=21,
+                         scale=0.5, softcap=2.0, width=32, blocks=1, conv=4,
+                         mlp=None),
+        O.delta_layer(heads=3, kv_heads=3, dim=8, vdim=8, conv=4,
+                      mlp=O.moe(5, 3, 16)),
+    ], width=64, vocab=48)
+
+
+def config_b():
+    # width not a multiple of 64, one tap, window 1, a single expert choice
+    return O.make_config([
+        O.parallel_layer(heads=3, kv_heads=1, dim=24, vdim=40, window=1,
+                         softcap=0.0, width=30, blocks=2, conv=1,
+                         mlp=O.moe(2, 2, 20)),
+        O.delta_layer(heads=4, kv_heads=2, dim=40, vdim=12, conv=2,
+                      mlp=None),
+        O.parallel_layer(heads=2, kv_heads=1, dim=16, vdim=16, window=37,
+                         width=96, blocks=4, conv=3, mlp=O.moe(6, 1, 8)),
+    ], width=96, vocab=70, embed_scale=0.5, eps=1e-6)
+
+
+CONFIGS = {"a": config_a, "b": config_b}
+_CKPT = {}
+
+
+def checkpoint(tmp_path_factory, name, slow_decay=False):
+    key = (name, slow_decay)
+    if key not in _CKPT:
+        cfg = CONFIGS[name]()
+        W = O.random_weights(cfg, seed=len(name) + 7 * slow_decay,
+                             slow_decay=slow_decay)
+        folder = O.write_checkpoint(
+            str(tmp_path_factory.mktemp(f"ckpt_{name}_{int(slow_decay)}")),
+            cfg, W)
+        _CKPT[key] = (cfg, W, folder)
+    return _CKPT[key]
+
+
+def engine(folder, mode, max_tokens=512, max_live=4):
+    from kaito_amd.engine.trace_replay import build_engine
+    device, dtype = mode
+    return build_engine(folder, dtype, max_tokens, device, max_live)
+
+
+def tokens(cfg, n, seed):
+    rng = random.Random(seed)
+    return [rng.randrange(cfg["vocab"]) for _ in range(n)]
+
+
+def row_err(got, want):
+    """Mean-free RMS difference per row relative to the oracle's logit
+    spread."""
+    d = got.double().cpu() - want
+    d = d - d.mean(-1, keepdim=True)
+    spread = (want - want.mean(-1, keepdim=True)).pow(2).mean().sqrt()
+    return (d.pow(2).mean(-1).sqrt() / spread).max().item()
+
+
+def tol(mode):
+    return 2e-4 if mode[1] == "float32" else 0.12
+
+
+def run_portions(eng, sid, toks, sizes):
+    """Feed toks to request sid in portions; returns all-row logits."""
+    out, at = [], 0
+    for n in sizes:
+        eng.extend_request(sid, toks[at:at + n])
+        out.append(eng.step_explicit([(sid, n)], [(0, i) for i in range(n)]))
+        at += n
+    assert at == len(toks)
+    return torch.cat(out, 0)
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_whole_prompt(tmp_path_factory, name, mode):
+    cfg, W, folder = checkpoint(tmp_path_factory, name)
+    toks = tokens(cfg, 45, 1)
+    want = O.model_logits(cfg, W, toks)
+    eng = engine(folder, mode)
+    got = run_portions(eng, 0, toks, [45])
+    assert row_err(got, want) < tol(mode)
+    # a one-token prompt: position 0 alone, nothing before it
+    got1 = run_portions(eng, 1, toks[:1], [1])
+    assert row_err(got1, want[:1]) < tol(mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_residual_stream_per_layer(tmp_path_factory, mode):
+    cfg, W, folder = checkpoint(tmp_path_factory, "a")
+    toks = tokens(cfg, 20, 2)
+    streams = []
+    O.model_logits(cfg, W, toks, streams)
+    eng = engine(folder, mode)
+    seen = []
+    eng.runner.model.layer_hook = lambda i, x: seen.append(x.clone())
+    run_portions(eng, 0, toks, [20])
+    lim = 1e-4 if mode[1] == "float32" else 0.1
+    for got, want in zip(seen, streams):
+        err = (got.double().cpu() - want).abs().max() / want.abs().max()
+        assert err < lim
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_decode_and_portions_match_whole(tmp_path_factory, name, mode):
+    cfg, W, folder = checkpoint(tmp_path_factory, name)
+    toks = tokens(cfg, 60, 3)
+    want = O.model_logits(cfg, W, toks)
+    eng = engine(folder, mode)
+    # prompt then one by one, far past every window and over page borders
+    got = run_portions(eng, 0, toks, [9] + [1] * 51)
+    assert row_err(got, want) < tol(mode)
+    # all one by one from the very first token
+    got = run_portions(eng, 1, toks, [1] * 60)
+    assert row_err(got, want) < tol(mode)
+    # uneven portions: 2-token ones, page-edge and window-edge cuts
+    got = run_portions(eng, 2, toks, [2, 2, 12, 1, 15, 2, 3, 11, 10, 2])
+    assert row_err(got, want) < tol(mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_unequal_batches_and_reuse(tmp_path_factory, mode):
+    """Requests of different lengths share steps (portions beside single
+    tokens); the page pool and the four state slots are too small for all
+    of them at once, so both are freed and used again."""
+    cfg, W, folder = checkpoint(tmp_path_factory, "a")
+    lens = [37, 5, 50, 18, 1, 33, 26]
+    reqs = [tokens(cfg, n, 10 + i) for i, n in enumerate(lens)]
+    want = [O.model_logits(cfg, W, t) for t in reqs]
+    eng = engine(folder, mode, max_tokens=192, max_live=4)
+    rng = random.Random(5)
+    at = [0] * len(reqs)
+    got = [[] for _ in reqs]
+    live, nxt = [], 0
+    while nxt < len(reqs) or live:
+        while nxt < len(reqs) and len(live) < 4 and \
+                sum(-(-lens[i] // 64) * 64 for i in live + [nxt]) <= 192:
+            live.append(nxt)
+            nxt += 1
+        portions, want_rows, owners = [], [], []
+        for i in list(live):
+            if rng.random() < 0.25 and len(live) > 1:
+                continue                      # sits this step out
+            left = lens[i] - at[i]
+            n = min(left, rng.choice([1, 1, 2, 3, 8, 17]))
+            eng.extend_request(i, reqs[i][at[i]:at[i] + n])
+            want_rows += [(len(portions), k) for k in range(n)]
+            owners += [i] * n
+            portions.append((i, n))
+            at[i] += n
+        if not portions:
+            continue
+        lg = eng.step_explicit(portions, want_rows)
+        for row, i in zip(lg, owners):
+            got[i].append(row)
+        for i in list(live):
+            if at[i] == lens[i]:
+                eng.release(i)
+                live.remove(i)
+    assert eng.pool.num_free == eng.pool.num_blocks
+    assert eng.state_pool.num_free == 4
+    for g, w in zip(got, want):
+        assert row_err(torch.stack(g), w) < tol(mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_far_tokens_reach_the_end(tmp_path_factory, mode):
+    """With slowly decaying recurrences the first token still moves the
+    logits 150 tokens later (far outside every attention window); the
+    engine must carry that through portions and decoding."""
+    cfg, W, folder = checkpoint(tmp_path_factory, "a", slow_decay=True)
+    toks = tokens(cfg, 150, 4)
+    other = [(toks[0] + 1) % cfg["vocab"]] + toks[1:]
+    want, want_other = (O.model_logits(cfg, W, t)[-8:] for t in (toks, other))
+    assert row_err(want_other.float(), want) > 20 * tol(mode), \
+        "the oracle itself must depend on the far token"
+    eng = engine(folder, mode)
+    got = run_portions(eng, 0, toks, [64, 2, 40, 30] + [1] * 14)[-8:]
+    assert row_err(got, want) < tol(mode)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_greedy_generation_through_scheduler(tmp_path_factory, mode):
+    """LLMEngine.generate (scheduler admission, prefill, batched decode,
+    sampler) against greedy decoding with the oracle."""
+    from kaito_amd.engine import SamplingParams
+    cfg, W, folder = checkpoint(tmp_path_factory, "a")
+    prompts = [tokens(cfg, n, 20 + n) for n in (5, 23, 1)]
+    eng = engine(folder, mode, max_tokens=512, max_live=4)
+    outs = eng.generate(prompts, SamplingParams(max_tokens=14,
+                                                ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        seq = list(p)
+        for tok in o.output_token_ids:
+            lg = O.model_logits(cfg, W, seq)[-1]
+            top2 = torch.topk(lg, 2).values
+            if mode[1] == "bfloat16" and top2[0] - top2[1] < 0.5:
+                break            # a near-tie may flip under bf16 rounding
+            assert tok == int(lg.argmax())
+            seq.append(tok)
+    assert eng.state_pool.num_free == 4
