@@ -142,12 +142,13 @@ def gurapel_model_config(cfg: dict, name: str = "",
 
 def layer_moe_config(cfg: ModelConfig, moe: MoESpec) -> ModelConfig:
     """A per-layer view of cfg for MoEMLP (layers may differ in expert
-    count, top-k and width). The expert width is rounded up to the fused
-    grouped-GEMM kernels' 64-column tile; the loader zero-fills the extra
-    gate/up rows and down columns, which contribute exactly nothing
-    (silu(0)·0 = 0)."""
+    count, top-k and width). For bf16 the expert width is rounded up to
+    the 64-column tile of the fused grouped-GEMM kernels (which also keeps
+    the vectorised activation kernel's alignment on the per-expert path);
+    the loader zero-fills the extra gate/up rows and down columns, which
+    contribute exactly nothing (silu(0)·0 = 0)."""
     ff = moe.ff
-    if cfg.hidden_size % 64 == 0 and cfg.dtype == torch.bfloat16:
+    if cfg.dtype == torch.bfloat16:
         ff = (ff + 63) // 64 * 64
     return dataclasses.replace(
         cfg, num_experts=moe.experts, num_experts_per_tok=moe.top,
