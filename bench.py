@@ -52,6 +52,18 @@ def parse_args():
                    metavar="OUT_CSV",
                    help="run TunableOp GEMM tuning for all decode shapes, "
                         "write results (default: in-tree csv), then exit")
+    p.add_argument("--hybrid-compare", default=None, nargs="?", const="all",
+                   metavar="SIZES",
+                   help="instead of the headline workload: prefill and "
+                        "decode tokens/s of the hybrid (Gurapel) stack "
+                        "beside the sliding-window MoE transformer of equal "
+                        "size, random weights; comma-separated sizes of "
+                        "kaito_amd.engine.hybrid_bench.SIZES (default all), "
+                        "one JSON line per size and model")
+    p.add_argument("--hybrid-batch", type=int, default=32)
+    p.add_argument("--hybrid-prompt", type=int, default=2048)
+    p.add_argument("--hybrid-out", type=int, default=128)
+    p.add_argument("--hybrid-models", default="gurapel,swa-moe")
     p.add_argument("--profile", action="store_true",
                    help="skip barriers/json (for rocprofv3 single-rank runs)")
     return p.parse_args()
@@ -68,6 +80,15 @@ def main():
     from kaito_amd.engine import EngineConfig, LLMEngine, SamplingParams
     from kaito_amd.models import get_model_config
     from kaito_amd.parallel import state as ps
+
+    if args.hybrid_compare is not None:
+        from kaito_amd.engine import hybrid_bench
+        sizes = list(hybrid_bench.SIZES) if args.hybrid_compare == "all" \
+            else args.hybrid_compare.split(",")
+        hybrid_bench.run(sizes, args.hybrid_batch, args.hybrid_prompt,
+                         args.hybrid_out, eager=args.eager,
+                         models=tuple(args.hybrid_models.split(",")))
+        return
 
     ps.init_parallel(tp_size=args.tp)
     st = ps.get_state()

@@ -1,0 +1,133 @@
+"""Prefill and decode throughput of the hybrid (Gurapel) stack beside the
+engine's closest homogeneous model at equal size: a sliding-window GQA
+transformer with the same MoE feed-forward (the gpt-oss class without
+sinks). Random weights, synthetic tokens; both models run through the
+same LLMEngine (scheduler, paged cache, hipGraph decode).
+
+Used by `bench.py --hybrid-compare`; prints one JSON line per
+(size, model).
+"""
+from __future__ import annotations
+
+import json
+import time
+from typing import Dict, List
+
+import torch
+
+# layers of a size: the hybrid pattern is delta, parallel, parallel
+SIZES: Dict[str, dict] = {
+    "w1024": dict(width=1024, layers=6, heads=8, kv_heads=2, dim=128,
+                  window=512, experts=8, top=2, ff=1024, vocab=32000,
+                  lru_blocks=8),
+    "w2048": dict(width=2048, layers=6, heads=16, kv_heads=4, dim=128,
+                  window=1024, experts=8, top=2, ff=2048, vocab=32000,
+                  lru_blocks=16),
+    "w4096": dict(width=4096, layers=6, heads=32, kv_heads=8, dim=128,
+                  window=1024, experts=8, top=2, ff=4096, vocab=32000,
+                  lru_blocks=16),
+}
+
+
+def hybrid_config(name: str, z: dict, max_pos: int):
+    from ..models.hybrid_config import gurapel_model_config
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]},
+           "router": {"experts": z["experts"], "top": z["top"]}}
+    delta = {"type": "delta", "mlp": moe, "mixer": {
+        "heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"],
+        "vdim": z["dim"], "conv": 4}}
+    par = {"type": "parallel", "mlp": moe, "mixer": {
+        "left": {"heads": z["heads"], "kv_heads": z["kv_heads"],
+                 "dim": z["dim"], "vdim": z["dim"],
+                 "mask": {"size": z["window"]}, "scale": z["dim"] ** -0.5,
+                 "softcap": 30.0},
+        "right": {"width": z["width"], "blocks": z["lru_blocks"],
+                  "conv": 4}}}
+    layers = [(delta if i % 3 == 0 else par) for i in range(z["layers"])]
+    return gurapel_model_config({
+        "architecture": "Gurapel", "embedding": {"scale": 1.0},
+        "layers": layers, "max_positions": max_pos, "norm": {"eps": 1e-5},
+        "vocab": z["vocab"], "width": z["width"]}, name=f"gurapel-{name}")
+
+
+def transformer_config(name: str, z: dict, max_pos: int):
+    from .config import ModelConfig
+    return ModelConfig(
+        name=f"swa-moe-{name}", hidden_size=z["width"],
+        num_layers=z["layers"], num_heads=z["heads"],
+        num_kv_heads=z["kv_heads"], head_dim=z["dim"],
+        intermediate_size=z["ff"], vocab_size=z["vocab"],
+        max_position=max_pos, num_experts=z["experts"],
+        num_experts_per_tok=z["top"], moe_intermediate_size=z["ff"],
+        moe_routing="topk_softmax", sliding_window=z["window"],
+        sliding_window_pattern="all")
+
+
+def _measure(mcfg, batch: int, prompt: int, out_tokens: int, eager: bool):
+    from .config import EngineConfig
+    from .engine import LLMEngine
+    from .sequence import SamplingParams
+    cfg = EngineConfig(
+        model=mcfg, device="cuda", max_num_seqs=batch,
+        max_model_len=prompt + out_tokens + 16,
+        max_num_batched_tokens=max(8192, prompt),
+        enforce_eager=eager, enable_prefix_caching=False,
+        graph_batch_sizes=(batch,), gpu_memory_utilization=0.5)
+    eng = LLMEngine(cfg)
+    if not eager:
+        eng.capture_graphs()
+    gen = torch.Generator().manual_seed(0)
+
+    def prompts():
+        return [torch.randint(10, mcfg.vocab_size - 10, (prompt,),
+                              generator=gen).tolist() for _ in range(batch)]
+
+    def one_round():
+        sp = SamplingParams(max_tokens=out_tokens, ignore_eos=True)
+        ids = [eng.add_request(p, sp) for p in prompts()]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while eng.scheduler.waiting or eng.scheduler.prefilling:
+            eng.step()
+        eng.flush()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        n0 = eng.num_generation_tokens
+        while eng.has_unfinished():
+            eng.step()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        n1 = eng.num_generation_tokens
+        for i in ids:
+            eng.seqs.pop(i, None)
+        return batch * prompt / (t1 - t0), (n1 - n0) / (t2 - t1)
+
+    one_round()                              # warm-up (allocator, GEMM pick)
+    pre, dec = zip(*(one_round() for _ in range(2)))
+    del eng
+    torch.cuda.empty_cache()
+    return max(pre), max(dec)
+
+
+def run(sizes: List[str], batch: int, prompt: int, out_tokens: int,
+        eager: bool = False, models=("gurapel", "swa-moe")) -> List[dict]:
+    from ..parallel import state as ps
+    ps.init_parallel(1)
+    results = []
+    for name in sizes:
+        z = SIZES[name]
+        max_pos = prompt + out_tokens + 16
+        for kind in models:
+            mcfg = hybrid_config(name, z, max_pos) if kind == "gurapel" \
+                else transformer_config(name, z, max_pos)
+            pre, dec = _measure(mcfg, batch, prompt, out_tokens, eager)
+            row = {"bench": "hybrid-compare", "size": name, "model": kind,
+                   "batch": batch, "prompt_tokens": prompt,
+                   "out_tokens": out_tokens,
+                   "prefill_tokens_per_s": round(pre, 1),
+                   "decode_tokens_per_s": round(dec, 1),
+                   "decode_graphs": not eager, "dtype": "bf16",
+                   "data": "synthetic"}
+            print(json.dumps(row), flush=True)
+            results.append(row)
+    return results

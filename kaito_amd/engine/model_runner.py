@@ -230,6 +230,12 @@ class ModelRunner:
                 [c.start for c in chunks], dtype=torch.int32, device=dev)
             meta.token_seq = torch.tensor(seq_of, dtype=torch.int32,
                                           device=dev)
+            if self.is_gpu and meta.max_seqlen >= 8:
+                # prompt portions: tile the chunks for the MFMA attention
+                # kernel (a step of single tokens keeps the decode kernel)
+                from .. import ops
+                meta.tile_seq, meta.tile_qbase = ops.build_query_tiles(
+                    [c.length for c in chunks], dev)
         if self.lora_manager is not None:
             tok_ids = []
             for c in chunks:

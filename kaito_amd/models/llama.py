@@ -44,6 +44,9 @@ class AttnMetadata:
     state_slots: Optional[torch.Tensor] = None   # [B] int32, <0 = padding
     seq_starts: Optional[torch.Tensor] = None    # [B] int32 first position
     token_seq: Optional[torch.Tensor] = None     # [T] int32 chunk of a row
+    # 64-row query tiles of the chunks (steps that hold prompt portions)
+    tile_seq: Optional[torch.Tensor] = None      # [tiles] int32
+    tile_qbase: Optional[torch.Tensor] = None    # [tiles] int32
 
 
 def build_cos_sin_cache(cfg: ModelConfig, device, max_pos: Optional[int] = None,

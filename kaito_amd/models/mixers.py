@@ -207,8 +207,12 @@ class BiasedWindowAttention(nn.Module):
         qn = ops.qk_norm_cache_write(q, k, v, self.q_norm, self.k_norm,
                                      self.norm_eps, cache["k"], cache["v"],
                                      meta.slot_mapping)
+        tiles = None
+        if meta.tile_seq is not None:
+            tiles = (meta.tile_seq, meta.tile_qbase, meta.cu_seqlens,
+                     meta.seq_starts)
         o = ops.window_attention(qn, cache["k"], cache["v"],
                                  meta.block_tables, meta.token_seq, positions,
                                  s.scale, s.softcap, self.r1, self.r2,
-                                 s.window)
+                                 s.window, tiles=tiles)
         return F.linear(o.reshape(T, -1), self.o_proj)

@@ -33,7 +33,8 @@ for _g, _names in {
     "comm": ("allreduce_rmsnorm one_shot_ar_rmsnorm ipc_handle ipc_open "
              "ipc_close"),
     "mix": ("causal_conv_update gated_delta_rule rglru_scan "
-            "qk_norm_cache_write window_attention post_norm_residual "
+            "qk_norm_cache_write window_attention window_attention_tiles "
+            "post_norm_residual "
             "rms_norm_cast"),
 }.items():
     for _n in _names.split():
@@ -440,17 +441,35 @@ def qk_norm_cache_write(q, k, v, q_w, k_w, eps: float, k_cache, v_cache,
                                          v_cache, slot_mapping)
 
 
+WINDOW_MFMA_SIZES = (64, 128, 256)
+
+
 def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
                      scale: float, softcap: float = 0.0, r1=None, r2=None,
-                     window: int = 0):
+                     window: int = 0, tiles=None):
     """Causal sliding-window attention of query rows [T, H, D] over the
     paged cache (key size D, value size V may differ), with optional tanh
     score capping and the distance penalty r1*ln(1 + r2*distance).
-    Returns [T, H, V]."""
+    Returns [T, H, V].
+
+    `tiles` = (tile_seq, tile_qbase, cu_seqlens, seq_starts) describes the
+    step's chunks as 64-row query tiles (build_query_tiles); with it, bf16
+    inputs of supported head sizes take the MFMA prompt kernel. Without
+    it (decode steps) or for f32 / other sizes, the one-row-per-workgroup
+    f32 kernel runs."""
     if q.is_cuda:
-        T, H, _ = q.shape
+        T, H, D = q.shape
         out = torch.empty(T, H, v_cache.size(3), dtype=q.dtype,
                           device=q.device)
+        if (tiles is not None and q.dtype == torch.bfloat16
+                and D in WINDOW_MFMA_SIZES
+                and v_cache.size(3) in WINDOW_MFMA_SIZES):
+            tile_seq, tile_qbase, cu, starts = tiles
+            _K.window_attention_tiles(
+                out, q, k_cache, v_cache, block_tables, tile_seq, tile_qbase,
+                cu, starts, scale, softcap, _none(r1, q), _none(r2, q),
+                window)
+            return out
         _K.window_attention(out, q, k_cache, v_cache, block_tables, token_seq,
                             positions, scale, softcap, _none(r1, q),
                             _none(r2, q), window)
@@ -458,6 +477,18 @@ def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
     return torch_ref.window_attention(q, k_cache, v_cache, block_tables,
                                       token_seq, positions, scale, softcap,
                                       r1, r2, window)
+
+
+def build_query_tiles(chunk_lens, device):
+    """Host-side tiling of a step's chunks into 64-row query tiles:
+    (tile_seq, tile_qbase) int32 tensors."""
+    seqs, bases = [], []
+    for i, n in enumerate(chunk_lens):
+        for q0 in range(0, n, QTILE):
+            seqs.append(i)
+            bases.append(q0)
+    return (torch.tensor(seqs, dtype=torch.int32, device=device),
+            torch.tensor(bases, dtype=torch.int32, device=device))
 
 
 def post_norm_residual(x32, y, w, eps: float, out_dtype, y2=None, w_y=None,

@@ -208,6 +208,182 @@ __global__ void window_attention_kernel(
   }
 }
 
+// ---- MFMA prompt-portion kernel (bf16) -------------------------------------
+// One workgroup = 64 query rows of one chunk x one head; 4 waves x 16 rows.
+// Keys come 32 at a time through LDS: the K tile XOR-swizzled for
+// conflict-free 16-byte fragment reads, the V tile transposed so the P.V
+// B-fragments are contiguous. S = Q K^T and O += P V run on
+// v_mfma_f32_16x16x32_bf16; scaling, capping, the distance penalty, the
+// window/causal mask and the online softmax are f32 on the accumulator
+// fragments. Key and value sizes are separate template parameters.
+constexpr int WQ_TILE = 64;
+constexpr int WKV_TILE = 32;
+constexpr int WPAD = 40;
+
+template <int D, int DV>
+__global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
+    short* __restrict__ out,              // [T, H, DV]
+    const short* __restrict__ q,          // [T, H, D]
+    const short* __restrict__ k_cache,    // [blocks, G, BS, D]
+    const short* __restrict__ v_cache,    // [blocks, G, BS, DV]
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_qbase,
+    const int* __restrict__ cu, const int* __restrict__ starts,
+    const int* __restrict__ block_tables, const int max_blocks,
+    const float scale, const float softcap, const float* __restrict__ r1,
+    const float* __restrict__ r2, const int window, const int H, const int G,
+    const int BS) {
+  constexpr int KK = D / 32;
+  constexpr int DT = DV / 16;
+  const int tile = blockIdx.x;
+  const int h = blockIdx.y;
+  const int g = h / (H / G);
+  const int seq = tile_seq[tile];
+  const int q0 = tile_qbase[tile];
+  const int tok0 = cu[seq];
+  const int q_len = cu[seq + 1] - tok0;
+  const int q_abs0 = starts[seq];          // position of the chunk's row 0
+  const int kv_len = q_abs0 + q_len;
+  const int* bt = block_tables + (int64_t)seq * max_blocks;
+  const float hr1 = r1 ? r1[h] : 0.f, hr2 = r1 ? r2[h] : 0.f;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int hi = lane >> 4;
+  const int lo = lane & 15;
+
+  __shared__ short lds_k[WKV_TILE * D];
+  __shared__ short lds_vt[DV * WPAD];
+  __shared__ short lds_p[4][16 * WPAD];
+
+  const int qrow = q0 + wave * 16 + lo;
+  const int qtok = tok0 + (qrow < q_len ? qrow : q_len - 1);
+  bf16x8 qfrag[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++)
+    qfrag[kk] = *reinterpret_cast<const bf16x8*>(
+        q + ((int64_t)qtok * H + h) * D + kk * 32 + hi * 8);
+
+  float mrow[4], lrow[4];
+  f32x4 ofrag[DT];
+#pragma unroll
+  for (int r = 0; r < 4; r++) { mrow[r] = -1e30f; lrow[r] = 0.f; }
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++) ofrag[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int kv_end = min(kv_len, q_abs0 + q0 + WQ_TILE);
+  const int kv_begin = (window > 0 && q_abs0 + q0 - window + 1 > 0)
+      ? ((q_abs0 + q0 - window + 1) / WKV_TILE) * WKV_TILE : 0;
+  for (int kv0 = kv_begin; kv0 < kv_end; kv0 += WKV_TILE) {
+    for (int i = threadIdx.x; i < WKV_TILE * D / 8; i += 256) {
+      const int row = (i * 8) / D;
+      const int col = (i * 8) % D;
+      const int kvp = min(kv0 + row, kv_len - 1);
+      const int64_t src =
+          (((int64_t)bt[kvp / BS] * G + g) * BS + (kvp % BS)) * D + col;
+      const short8_t kd = *reinterpret_cast<const short8_t*>(k_cache + src);
+      const int swz = (col * 2) ^ ((row & 7) << 4);
+      *reinterpret_cast<short8_t*>(&lds_k[row * D + swz / 2]) = kd;
+    }
+    for (int i = threadIdx.x; i < WKV_TILE * DV / 8; i += 256) {
+      const int row = (i * 8) / DV;
+      const int col = (i * 8) % DV;
+      const int kvp = min(kv0 + row, kv_len - 1);
+      const int64_t src =
+          (((int64_t)bt[kvp / BS] * G + g) * BS + (kvp % BS)) * DV + col;
+      const short8_t vd = *reinterpret_cast<const short8_t*>(v_cache + src);
+#pragma unroll
+      for (int j = 0; j < 8; j++) lds_vt[(col + j) * WPAD + row] = vd[j];
+    }
+    __syncthreads();
+
+    f32x4 sfrag[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++) {
+      sfrag[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) {
+        const int krow = kt * 16 + lo;
+        const int swz = ((kk * 32 + hi * 8) * 2) ^ ((krow & 7) << 4);
+        const bf16x8 kf =
+            *reinterpret_cast<const bf16x8*>(&lds_k[krow * D + swz / 2]);
+        sfrag[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            qfrag[kk], kf, sfrag[kt], 0, 0, 0);
+      }
+    }
+
+    float p[2][4];
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int qr = q0 + wave * 16 + hi * 4 + r;
+        const int q_abs = q_abs0 + qr;
+        const int kvp = kv0 + kt * 16 + lo;
+        float sv = sfrag[kt][r] * scale;
+        if (softcap > 0.f)          // cap * tanh(s / cap), via exp
+          sv = softcap * (1.0f - 2.0f / (__expf(2.0f * sv * inv_cap) + 1.0f));
+        const int dist = q_abs - kvp;
+        if (r1) sv -= hr1 * __logf(1.0f + hr2 * (float)max(dist, 0));
+        if (dist < 0 || kvp >= kv_len || qr >= q_len ||
+            (window > 0 && dist >= window)) sv = -1e30f;
+        p[kt][r] = sv;
+      }
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      float mx = fmaxf(p[0][r], p[1][r]);
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+      const float mnew = fmaxf(mrow[r], mx);
+      const float corr = __expf(mrow[r] - mnew);
+      lrow[r] *= corr;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) ofrag[dt][r] *= corr;
+      mrow[r] = mnew;
+      float ps = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++) {
+        p[kt][r] = __expf(p[kt][r] - mnew);
+        ps += p[kt][r];
+      }
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) ps += __shfl_xor(ps, off, 64);
+      lrow[r] += ps;
+    }
+    {
+      short* pl = lds_p[wave];
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          pl[(hi * 4 + r) * WPAD + kt * 16 + lo] = f32_to_bf16(p[kt][r]);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    const bf16x8 pfrag = *reinterpret_cast<const bf16x8*>(
+        &lds_p[wave][lo * WPAD + hi * 8]);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      const bf16x8 vf = *reinterpret_cast<const bf16x8*>(
+          &lds_vt[(dt * 16 + lo) * WPAD + hi * 8]);
+      ofrag[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pfrag, vf,
+                                                          ofrag[dt], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const int qr = q0 + wave * 16 + hi * 4 + r;
+    if (qr >= q_len) continue;
+    const float inv = 1.f / fmaxf(lrow[r], 1e-30f);
+    const int64_t obase = ((int64_t)(tok0 + qr) * H + h) * DV;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+      out[obase + dt * 16 + lo] = f32_to_bf16(ofrag[dt][r] * inv);
+  }
+}
+
 }  // namespace
 
 void qk_norm_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor k,
@@ -299,13 +475,73 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
   });
 }
 
+// Prompt-portion path: 64-row query tiles (tile_seq[i] = chunk, tile_qbase[i]
+// = first row of the tile inside its chunk) on the MFMA kernel. bf16 with
+// key/value sizes from {64, 128, 256}; callers fall back to
+// window_attention otherwise (see window_attention_tiles_supported).
+void window_attention_tiles(at::Tensor out, at::Tensor q, at::Tensor k_cache,
+                            at::Tensor v_cache, at::Tensor block_tables,
+                            at::Tensor tile_seq, at::Tensor tile_qbase,
+                            at::Tensor cu_seqlens, at::Tensor seq_starts,
+                            double scale, double softcap, at::Tensor r1,
+                            at::Tensor r2, int64_t window) {
+  TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() &&
+              q.dtype() == at::kBFloat16);
+  const int T = q.size(0), H = q.size(1), D = q.size(2);
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.dtype() == q.dtype() && v_cache.dtype() == q.dtype());
+  const int G = k_cache.size(1), BS = k_cache.size(2), V = v_cache.size(3);
+  TORCH_CHECK(k_cache.size(3) == D && v_cache.size(1) == G &&
+              v_cache.size(2) == BS && H % G == 0);
+  TORCH_CHECK(out.is_contiguous() && out.dtype() == q.dtype() &&
+              out.dim() == 3 && out.size(0) == T && out.size(1) == H &&
+              out.size(2) == V);
+  KAITO_CHECK_I32(block_tables); KAITO_CHECK_I32(tile_seq);
+  KAITO_CHECK_I32(tile_qbase); KAITO_CHECK_I32(cu_seqlens);
+  KAITO_CHECK_I32(seq_starts);
+  TORCH_CHECK(block_tables.dim() == 2 &&
+              tile_qbase.size(0) == tile_seq.size(0) &&
+              cu_seqlens.size(0) == seq_starts.size(0) + 1 &&
+              block_tables.size(0) >= seq_starts.size(0));
+  const bool bias = r1.numel() > 0;
+  if (bias) {
+    KAITO_CHECK_F32(r1); KAITO_CHECK_F32(r2);
+    TORCH_CHECK(r1.numel() == H && r2.numel() == H);
+  }
+  const int ntiles = tile_seq.size(0);
+  if (ntiles == 0 || T == 0) return;
+  auto stream = at::hip::getCurrentHIPStream();
+#define KAITO_WIN_CASE(D_, DV_)                                              \
+  if (D == D_ && V == DV_) {                                                 \
+    hipLaunchKernelGGL((window_attention_mfma_kernel<D_, DV_>),              \
+        dim3(ntiles, H), dim3(256), 0, stream, (short*)out.data_ptr(),       \
+        (const short*)q.data_ptr(), (const short*)k_cache.data_ptr(),        \
+        (const short*)v_cache.data_ptr(), tile_seq.data_ptr<int>(),          \
+        tile_qbase.data_ptr<int>(), cu_seqlens.data_ptr<int>(),              \
+        seq_starts.data_ptr<int>(), block_tables.data_ptr<int>(),            \
+        (int)block_tables.size(1), (float)scale, (float)softcap,             \
+        bias ? r1.data_ptr<float>() : nullptr,                               \
+        bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, BS);       \
+    return;                                                                  \
+  }
+  KAITO_WIN_CASE(64, 64) KAITO_WIN_CASE(64, 128) KAITO_WIN_CASE(128, 64)
+  KAITO_WIN_CASE(128, 128) KAITO_WIN_CASE(128, 256) KAITO_WIN_CASE(256, 128)
+  KAITO_WIN_CASE(256, 256) KAITO_WIN_CASE(64, 256) KAITO_WIN_CASE(256, 64)
+#undef KAITO_WIN_CASE
+  TORCH_CHECK(false, "window_attention_tiles: key/value sizes must be from "
+              "{64, 128, 256}, got ", D, "/", V);
+}
+
 }  // namespace kaito
 
 TORCH_LIBRARY_FRAGMENT(kaito, m) {
+  m.def("window_attention_tiles(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor tile_seq, Tensor tile_qbase, Tensor cu_seqlens, Tensor seq_starts, float scale, float softcap, Tensor r1, Tensor r2, int window) -> ()");
   m.def("qk_norm_cache_write(Tensor(a!) q_out, Tensor q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, float eps, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slot_mapping) -> ()");
   m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor token_seq, Tensor positions, float scale, float softcap, Tensor r1, Tensor r2, int window) -> ()");
 }
 TORCH_LIBRARY_IMPL(kaito, CUDA, m) {
   m.impl("qk_norm_cache_write", &kaito::qk_norm_cache_write);
   m.impl("window_attention", &kaito::window_attention);
+  m.impl("window_attention_tiles", &kaito::window_attention_tiles);
 }

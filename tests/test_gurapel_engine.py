@@ -50,7 +50,20 @@ def config_b():
     ], width=96, vocab=70, embed_scale=0.5, eps=1e-6)
 
 
-CONFIGS = {"a": config_a, "b": config_b}
+def config_c():
+    # head sizes the tiled MFMA prompt kernel takes (bf16), width a
+    # multiple of 64 so the fused MoE kernels run too
+    return O.make_config([
+        O.parallel_layer(heads=2, kv_heads=1, dim=64, vdim=128, window=19,
+                         width=64, blocks=2, conv=4, mlp=O.moe(4, 2, 48)),
+        O.delta_layer(heads=2, kv_heads=1, dim=64, vdim=32, conv=4,
+                      mlp=O.moe(4, 2, 64)),
+        O.parallel_layer(heads=2, kv_heads=2, dim=128, vdim=64, window=40,
+                         softcap=8.0, width=128, blocks=1, conv=2, mlp=None),
+    ], width=128, vocab=64)
+
+
+CONFIGS = {"a": config_a, "b": config_b, "c": config_c}
 _CKPT = {}
 
 
@@ -147,7 +160,7 @@ def test_residual_stream_per_layer(tmp_path_factory, mode):
 
 
 @pytest.mark.parametrize("mode", MODES)
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
 def test_decode_and_portions_match_whole(tmp_path_factory, name, mode):
     cfg, W, folder = checkpoint(tmp_path_factory, name)
     toks = tokens(cfg, 60, 3)

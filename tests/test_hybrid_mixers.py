@@ -337,3 +337,72 @@ def test_moe_router_and_experts(mode, experts, top, ff, width):
     want = O.moe_ff(x.double(), {"p." + k: v.double() for k, v in W.items()},
                     "p.", cfg["layers"][0]["mlp"])
     close(mlp(x.to(dev)), want, dt)
+
+
+# ------------------------------------------- MFMA prompt-portion attention
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,V,window", [(4, 1, 64, 128, 96),
+                                            (2, 2, 128, 64, 70),
+                                            (2, 1, 64, 64, 0),
+                                            (4, 2, 128, 128, 33),
+                                            (1, 1, 256, 256, 130)])
+def test_window_attention_tiled_prompt_kernel(H, G, D, V, window):
+    """Several chunks of one step (fresh prompts, continued portions that
+    start inside a page and inside a window, a single token) on the tiled
+    MFMA kernel against the plain attention."""
+    dev, dt = "cuda", torch.bfloat16
+    # (start, length): history before `start` is fed by an earlier step
+    chunks = [(0, 150), (37, 70), (200, 1), (5, 64), (130, 3)]
+    r1, r2 = torch.rand(H), torch.rand(H) * 2
+    n_pages = sum(-(-(s + n) // BS) for s, n in chunks) + 1
+    kc, vc = paged(dev, dt, G, D, V, n_pages)
+    free = list(range(n_pages))[::-1]
+    seqs, tables = [], []
+    for s, n in chunks:
+        T = s + n
+        q = torch.randn(T, H, D).to(dt)
+        k = torch.randn(T, G, D).to(dt)
+        v = torch.randn(T, G, V).to(dt)
+        pages = [free.pop() for _ in range(-(-T // BS))]
+        seqs.append((q, k, v, pages))
+        tables.append(pages)
+    mb = max(len(p) for p in tables)
+    bt = torch.tensor([p + [0] * (mb - len(p)) for p in tables],
+                      dtype=torch.int32, device=dev)
+
+    def slots(pages, a, b):
+        return torch.tensor([pages[p // BS] * BS + p % BS
+                             for p in range(a, b)], dtype=torch.long,
+                            device=dev)
+
+    # step 1: histories, each sequence alone (no norm weights: plain write)
+    for (s, n), (q, k, v, pages) in zip(chunks, seqs):
+        if s:
+            ops.qk_norm_cache_write(q[:s].to(dev), k[:s].to(dev),
+                                    v[:s].to(dev), None, None, 1e-5, kc, vc,
+                                    slots(pages, 0, s))
+    # step 2: all chunks together
+    cu, sl, st, ts, pos = layout(dev, [n for _, n in chunks],
+                                 [s for s, _ in chunks],
+                                 list(range(len(chunks))))
+    qs = torch.cat([q[s:s + n] for (s, n), (q, _, _, _) in zip(chunks, seqs)])
+    ks = torch.cat([k[s:s + n] for (s, n), (_, k, _, _) in zip(chunks, seqs)])
+    vs = torch.cat([v[s:s + n] for (s, n), (_, _, v, _) in zip(chunks, seqs)])
+    sm = torch.cat([slots(p, s, s + n)
+                    for (s, n), (_, _, _, p) in zip(chunks, seqs)])
+    qn = ops.qk_norm_cache_write(qs.to(dev), ks.to(dev), vs.to(dev), None,
+                                 None, 1e-5, kc, vc, sm)
+    tiles = ops.build_query_tiles([n for _, n in chunks], dev) + (cu, st)
+    got = ops.window_attention(qn, kc, vc, bt, ts, pos, 0.1, 4.0,
+                               r1.to(dev), r2.to(dev), window, tiles=tiles)
+    plain = ops.window_attention(qn, kc, vc, bt, ts, pos, 0.1, 4.0,
+                                 r1.to(dev), r2.to(dev), window)
+    at = 0
+    for (s, n), (q, k, v, _) in zip(chunks, seqs):
+        want = O.window_attention(q.double(), k.double(), v.double(),
+                                  window or s + n, 0.1, 4.0, r1.double(),
+                                  r2.double())[s:]
+        close(got[at:at + n], want, dt)
+        close(plain[at:at + n], want, dt)
+        at += n
