@@ -148,7 +148,8 @@ class RGLRUMixer(nn.Module):
         ub = u.float().view(T, s.blocks, self.bw).transpose(0, 1)
         gates = torch.baddbmm(self.gate_b, ub, self.gate_w)   # [B, T, 2bw]
         o = ops.rglru_scan(u, gates, p[:, :w], self.decay_rate, cache["lru"],
-                           meta.cu_seqlens, meta.state_slots, meta.seq_starts)
+                           meta.cu_seqlens, meta.state_slots, meta.seq_starts,
+                           meta.token_seq)
         return F.linear(o, self.o_proj)
 
 

@@ -414,14 +414,17 @@ def gated_delta_rule(q, k, v, gate, a, b, a_log, dt_bias, norm_w, state,
 
 
 def rglru_scan(u, gates, y, decay_rate, state, cu_seqlens, state_slots,
-               seq_starts):
+               seq_starts, token_seq=None):
     """Real-gated linear recurrence + GELU gate branch. u/y [T, W] (row
     strides free); gates [B, T, 2*W/B] f32; decay_rate [W] f32; state
     [slots, W] f32 in place. Returns [T, W]."""
     if u.is_cuda:
         out = torch.empty(u.shape, dtype=u.dtype, device=u.device)
+        # with token_seq, prompt-sized steps take the segment-parallel scan
         _K.rglru_scan(out, u, gates, y, decay_rate, state, cu_seqlens,
-                      state_slots, seq_starts)
+                      state_slots, seq_starts,
+                      token_seq if token_seq is not None else
+                      torch.empty(0, dtype=torch.int32, device=u.device))
         return out
     return torch_ref.rglru_scan(u, gates, y, decay_rate, state, cu_seqlens,
                                 state_slots, seq_starts)

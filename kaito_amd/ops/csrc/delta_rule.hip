@@ -163,6 +163,149 @@ __global__ void delta_recurrence_kernel(
   }
 }
 
+// Wave-per-column-group recurrence (the fast path; dim % 4 == 0). The
+// columns of S are independent, so a (chunk, head) pair is split over
+// V / VB single-wave workgroups of VB = 64 / PARTS columns each: many
+// more waves in flight than one workgroup per head, no workgroup barrier
+// between waves, and the PARTS-wide sums are DPP butterflies. Token tiles
+// are double-buffered: the next tile's global loads are issued before the
+// current tile is consumed and parked in LDS afterwards. k and q rows are
+// zero-padded to DP * PARTS in LDS so the inner loops read unconditional
+// float4s; the dot products run on four independent accumulators.
+template <typename T, int DP, int PARTS>
+__global__ __launch_bounds__(64) void delta_recurrence_wave_kernel(
+    float* __restrict__ o,                                 // [T, H, V]
+    const float* __restrict__ qn, const float* __restrict__ kn,
+    const T* __restrict__ v, const int64_t v_s0, const int64_t v_s1,
+    const float* __restrict__ decay, const float* __restrict__ beta,
+    float* __restrict__ state,                             // [slots, H, D, V]
+    const int* __restrict__ cu, const int* __restrict__ slots,
+    const int* __restrict__ starts, const int G, const int D, const int H,
+    const int V) {
+  constexpr int TT = TOK_TILE;
+  constexpr int VB = 64 / PARTS;
+  constexpr int DPAD = DP * PARTS;
+  constexpr int ROW = 2 * DPAD + VB + 4;      // k | q | v | decay beta - -
+  constexpr int KQ4 = TT * DPAD / 4 / 64;     // float4 loads per lane
+  constexpr int VN = (TT * VB + 63) / 64;
+  __shared__ __attribute__((aligned(16))) float lds[2][TT * ROW];
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int slot = slots[b];
+  const int r0 = cu[b], r1 = cu[b + 1];
+  if (slot < 0 || r1 <= r0) return;
+  const int g = h / (H / G);
+  const int tid = threadIdx.x;
+  const int part = tid % PARTS;
+  const int jl = tid / PARTS;                 // column inside the group
+  const int j = blockIdx.z * VB + jl;
+  const bool live = j < V;
+  const int d0 = part * DP;
+  float S[DP];
+  float* sp = state + (((int64_t)slot * H + h) * D) * V + j;
+  const bool carried = starts[b] > 0;
+#pragma unroll
+  for (int i = 0; i < DP; i++) {
+    const int d = d0 + i;
+    S[i] = (carried && live && d < D) ? sp[(int64_t)d * V] : 0.0f;
+  }
+
+  float4_t rk[KQ4], rq[KQ4];
+  float rv[VN], rdb = 0.f;
+  auto fetch = [&](int t0) {
+    const int nt = min(TT, r1 - t0);
+#pragma unroll
+    for (int i = 0; i < KQ4; i++) {
+      const int e = tid + i * 64;
+      const int tt = e / (DPAD / 4), d = (e % (DPAD / 4)) * 4;
+      const bool ok = tt < nt && d < D;
+      const int64_t src = ((int64_t)(t0 + tt) * G + g) * D + d;
+      rk[i] = ok ? *reinterpret_cast<const float4_t*>(kn + src)
+                 : float4_t{0.f, 0.f, 0.f, 0.f};
+      rq[i] = ok ? *reinterpret_cast<const float4_t*>(qn + src)
+                 : float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int i = 0; i < VN; i++) {
+      const int e = tid + i * 64;
+      const int tt = e / VB, c = blockIdx.z * VB + e % VB;
+      rv[i] = (e < TT * VB && tt < nt && c < V)
+          ? act_ld(v + (int64_t)(t0 + tt) * v_s0 + (int64_t)h * v_s1 + c)
+          : 0.f;
+    }
+    if (tid < 2 * TT) {
+      const int tt = tid >> 1;
+      const float* src = (tid & 1) ? beta : decay;
+      rdb = tt < nt ? src[(int64_t)(t0 + tt) * H + h] : 0.f;
+    }
+  };
+  auto park = [&](float* buf) {
+#pragma unroll
+    for (int i = 0; i < KQ4; i++) {
+      const int e = tid + i * 64;
+      const int tt = e / (DPAD / 4), d = (e % (DPAD / 4)) * 4;
+      *reinterpret_cast<float4_t*>(buf + tt * ROW + d) = rk[i];
+      *reinterpret_cast<float4_t*>(buf + tt * ROW + DPAD + d) = rq[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VN; i++) {
+      const int e = tid + i * 64;
+      if (e < TT * VB) buf[(e / VB) * ROW + 2 * DPAD + e % VB] = rv[i];
+    }
+    if (tid < 2 * TT) buf[(tid >> 1) * ROW + 2 * DPAD + VB + (tid & 1)] = rdb;
+  };
+
+  fetch(r0);
+  park(lds[0]);
+  __syncthreads();
+  int cur = 0;
+  for (int t0 = r0; t0 < r1; t0 += TT) {
+    const int nt = min(TT, r1 - t0);
+    const bool more = t0 + TT < r1;
+    if (more) fetch(t0 + TT);
+    const float* buf = lds[cur];
+    for (int tt = 0; tt < nt; tt++) {
+      const float* lk = buf + tt * ROW + d0;
+      const float* lq = lk + DPAD;
+      const float dec = buf[tt * ROW + 2 * DPAD + VB];
+      const float bet = buf[tt * ROW + 2 * DPAD + VB + 1];
+      const float vj = buf[tt * ROW + 2 * DPAD + jl];
+      float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
+#pragma unroll
+      for (int i = 0; i < DP; i += 4) {
+        const float4_t k4 = *reinterpret_cast<const float4_t*>(lk + i);
+        S[i] *= dec; S[i + 1] *= dec; S[i + 2] *= dec; S[i + 3] *= dec;
+        p0 += S[i] * k4[0]; p1 += S[i + 1] * k4[1];
+        p2 += S[i + 2] * k4[2]; p3 += S[i + 3] * k4[3];
+      }
+      const float pred = group_reduce_sum<PARTS>((p0 + p1) + (p2 + p3));
+      const float u = bet * (vj - pred);
+      p0 = p1 = p2 = p3 = 0.f;
+#pragma unroll
+      for (int i = 0; i < DP; i += 4) {
+        const float4_t k4 = *reinterpret_cast<const float4_t*>(lk + i);
+        const float4_t q4 = *reinterpret_cast<const float4_t*>(lq + i);
+        S[i] += k4[0] * u; S[i + 1] += k4[1] * u;
+        S[i + 2] += k4[2] * u; S[i + 3] += k4[3] * u;
+        p0 += S[i] * q4[0]; p1 += S[i + 1] * q4[1];
+        p2 += S[i + 2] * q4[2]; p3 += S[i + 3] * q4[3];
+      }
+      const float oj = group_reduce_sum<PARTS>((p0 + p1) + (p2 + p3));
+      if (live && part == 0)
+        o[((int64_t)(t0 + tt) * H + h) * V + j] = oj;
+    }
+    if (more) park(lds[cur ^ 1]);
+    __syncthreads();
+    cur ^= 1;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < DP; i++) {
+      const int d = d0 + i;
+      if (d < D) sp[(int64_t)d * V] = S[i];
+    }
+  }
+}
+
 template <typename T>
 __global__ void delta_epilogue_kernel(
     T* __restrict__ out,                                   // [T, H*V]
@@ -226,9 +369,30 @@ void run_delta(hipStream_t stream, at::Tensor& out, const at::Tensor& q,
       (const T*)a.data_ptr(), a.stride(0), (const T*)b.data_ptr(),
       b.stride(0), a_log.data_ptr<float>(), dt_bias.data_ptr<float>(), G, D,
       H, qk_eps);
-  KAITO_DELTA_CASE(32, 1) KAITO_DELTA_CASE(32, 2) KAITO_DELTA_CASE(32, 4)
-  KAITO_DELTA_CASE(32, 8) KAITO_DELTA_CASE(64, 1) KAITO_DELTA_CASE(64, 2)
-  KAITO_DELTA_CASE(64, 4) KAITO_DELTA_CASE(64, 8)
+  int wparts = 1;
+  while (wparts * 32 < D) wparts <<= 1;
+  if (D % 4 == 0 && wparts <= 8) {
+    // fast path: single-wave workgroups over groups of 64 / PARTS columns
+#define KAITO_DELTA_WAVE(PARTS_)                                             \
+    if (wparts == PARTS_) {                                                  \
+      constexpr int VB = 64 / PARTS_;                                        \
+      hipLaunchKernelGGL((delta_recurrence_wave_kernel<T, 32, PARTS_>),      \
+          dim3(B, H, (V + VB - 1) / VB), dim3(64), 0, stream,                \
+          o.data_ptr<float>(), qn.data_ptr<float>(), kn.data_ptr<float>(),   \
+          (const T*)v.data_ptr(), v.stride(0), v.stride(1),                  \
+          decay.data_ptr<float>(), beta.data_ptr<float>(),                   \
+          state.data_ptr<float>(), cu_seqlens.data_ptr<int>(),               \
+          state_slots.data_ptr<int>(), seq_starts.data_ptr<int>(), G, D, H,  \
+          V);                                                                \
+    }
+    KAITO_DELTA_WAVE(1) KAITO_DELTA_WAVE(2) KAITO_DELTA_WAVE(4)
+    KAITO_DELTA_WAVE(8)
+#undef KAITO_DELTA_WAVE
+  } else {
+    KAITO_DELTA_CASE(32, 1) KAITO_DELTA_CASE(32, 2) KAITO_DELTA_CASE(32, 4)
+    KAITO_DELTA_CASE(32, 8) KAITO_DELTA_CASE(64, 1) KAITO_DELTA_CASE(64, 2)
+    KAITO_DELTA_CASE(64, 4) KAITO_DELTA_CASE(64, 8)
+  }
   hipLaunchKernelGGL((delta_epilogue_kernel<T>), dim3(T_, H), dim3(64), 0,
       stream, (T*)out.data_ptr(), o.data_ptr<float>(),
       (const T*)gate.data_ptr(), gate.stride(0), gate.stride(1),

@@ -90,7 +90,8 @@ def plain_delta(q, k, v, gate, a, b, a_log, dt_bias, norm_w, eps):
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("G,H,D,V", [(1, 2, 16, 24), (3, 3, 8, 8),
                                      (2, 4, 48, 40), (1, 1, 128, 64),
-                                     (1, 2, 64, 130)])
+                                     (1, 2, 64, 130), (1, 2, 10, 12),
+                                     (1, 1, 256, 20)])
 def test_delta_rule_portions(mode, G, H, D, V):
     dev, dt = mode
     T = 29
@@ -159,6 +160,44 @@ def test_rglru_portions_and_batch(mode, W, NB):
             at += n
     for g, w in zip(got, want):
         close(torch.cat(g), w, dt)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_rglru_prompt_sized_step(mode):
+    """A step of long portions (the segment-parallel scan on the GPU):
+    chunk borders inside segments, a carried state, a one-token chunk and
+    a padding chunk."""
+    dev, dt = mode
+    W, NB = 96, 2
+    bw = W // NB
+    lens, starts, slots = [150, 1, 70, 9, 130], [0, 5, 33, 0, 64], \
+        [2, 0, 1, -1, 3]
+    T = sum(lens)
+    u, y = torch.randn(T, W).to(dt), torch.randn(T, W).to(dt)
+    gates = torch.randn(NB, T, 2 * bw)
+    rate = torch.rand(W) * 0.2
+    init = torch.randn(4, W)
+    state = init.clone().to(dev)
+    cu, sl, st, ts, _ = layout(dev, lens, starts, slots)
+    got = ops.rglru_scan(u.to(dev), gates.to(dev), y.to(dev), rate.to(dev),
+                         state, cu, sl, st, ts)
+    g = gates.double().permute(1, 0, 2)
+    rg = torch.sigmoid(g[..., :bw]).reshape(T, W)
+    ig = torch.sigmoid(g[..., bw:]).reshape(T, W)
+    aa = torch.exp(-rg * rate.double())
+    at = 0
+    for n, s0, slot in zip(lens, starts, slots):
+        if slot >= 0:
+            S = init[slot].double() if s0 > 0 else torch.zeros(W,
+                                                               dtype=O.F64)
+            rows = []
+            for t in range(at, at + n):
+                S = aa[t] * S + torch.sqrt(1 - aa[t] ** 2) * ig[t] \
+                    * u[t].double()
+                rows.append(S * O.gelu_tanh(y[t].double()))
+            close(got[at:at + n], torch.stack(rows), dt)
+            close(state[slot], S, torch.float32)
+        at += n
 
 
 # --------------------------------------------------------------- attention
