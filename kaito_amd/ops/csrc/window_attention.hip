@@ -384,6 +384,251 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
   }
 }
 
+// ---- decode kernel: one workgroup per (query row, kv head) -----------------
+// All H/G query heads that share a kv head are served by one pass over its
+// K and V rows (up to RT heads per workgroup; more heads take further
+// passes on blockIdx.z). Per tile of up to KT keys:
+//   scores : a wave takes 8 keys at a time, 8 lanes per key, each lane
+//            16-byte chunks of the key row (contiguous 128 B per key); the
+//            lane's slices of the RT query rows live in registers; 8-lane
+//            DPP butterflies finish the dot products.
+//   softmax: wave r mod 4 owns head r: tile max, exp, sum, running max and
+//            sum with the rescale factor of the earlier tiles.
+//   P.V    : a wave takes every 4th key for all heads, a lane a slice of
+//            the value row (coalesced row reads), weights broadcast from
+//            LDS; the four waves' partial sums meet in LDS at the end.
+template <typename T, int RT, int NCH>
+__global__ __launch_bounds__(256) void window_attention_decode_kernel(
+    T* __restrict__ out, const T* __restrict__ q,
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_tables, const int max_blocks,
+    const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
+    const float scale, const float softcap, const float* __restrict__ r1,
+    const float* __restrict__ r2, const int window, const int H, const int G,
+    const int D, const int V, const int BS, const int KT) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  extern __shared__ float lds[];
+  float* s_s = lds;                            // [RT][KT]
+  int* row_s = reinterpret_cast<int*>(s_s + RT * KT);   // [KT]
+  float* m_s = reinterpret_cast<float*>(row_s + KT);    // [RT] running max
+  float* l_s = m_s + RT;                       // [RT] running sum
+  float* c_s = l_s + RT;                       // [RT] rescale of this tile
+  float* acc_s = c_s + RT;                     // [4][RT][256]
+
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int R = H / G;
+  const int rbase = blockIdx.z * RT;
+  const int nr = min(RT, R - rbase);
+  const int h0 = g * R + rbase;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int sub = lane & 7, kl = lane >> 3;    // chunk lane, key in the wave
+  const int b = token_seq[t];
+  if (b < 0) {
+    for (int r = 0; r < nr; r++)
+      for (int j = tid; j < V; j += 256)
+        act_st(out + ((int64_t)t * H + h0 + r) * V + j, 0.0f);
+    return;
+  }
+  const int pos = (int)positions[t];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int nkeys = pos - lo + 1;
+  const int* bt = block_tables + (int64_t)b * max_blocks;
+  const int nchunks = D / VEC;
+
+  float qreg[RT][NCH][VEC];
+#pragma unroll
+  for (int r = 0; r < RT; r++)
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      const int ch = sub + 8 * i;
+#pragma unroll
+      for (int e = 0; e < VEC; e++)
+        qreg[r][i][e] = (r < nr && ch < nchunks)
+            ? act_ld(q + ((int64_t)t * H + h0 + r) * D + ch * VEC + e) : 0.0f;
+    }
+  float hr1[RT], hr2[RT];
+#pragma unroll
+  for (int r = 0; r < RT; r++) {
+    hr1[r] = (r1 && r < nr) ? r1[h0 + r] : 0.0f;
+    hr2[r] = (r1 && r < nr) ? r2[h0 + r] : 0.0f;
+  }
+  // P.V lane roles: LPR lanes cover one value row in 16-byte chunks, so a
+  // wave load touches 64 / LPR rows at once
+  const int vchunks = V / VEC;
+  int lpr = 1;
+  while (lpr < vchunks) lpr <<= 1;
+  const int rpw = 64 / lpr;
+  const int vch = lane % lpr, rsub = lane / lpr;
+  const bool vlive = vch < vchunks;
+  float acc[RT][VEC];
+#pragma unroll
+  for (int r = 0; r < RT; r++)
+#pragma unroll
+    for (int e = 0; e < VEC; e++) acc[r][e] = 0.0f;
+  if (tid < RT) { m_s[tid] = -INFINITY; l_s[tid] = 0.0f; }
+
+  for (int k0 = 0; k0 < nkeys; k0 += KT) {
+    const int nk = min(KT, nkeys - k0);
+    __syncthreads();                 // previous tile's P.V done with s_s
+    // ---- scores: UNR key groups per trip, all their loads issued first
+    constexpr int UNR = 4;
+    for (int kb = wave * 8 + kl; kb < nk; kb += 32 * UNR) {
+      int rowi[UNR];
+      float kv[UNR][NCH][VEC];
+#pragma unroll
+      for (int un = 0; un < UNR; un++) {
+        const int j = lo + k0 + min(kb + 32 * un, nk - 1);
+        rowi[un] = (bt[j / BS] * G + g) * BS + (j % BS);
+      }
+#pragma unroll
+      for (int un = 0; un < UNR; un++) {
+        const T* krow = k_cache + (int64_t)rowi[un] * D;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+          const int ch = min(sub + 8 * i, nchunks - 1);
+          if constexpr (sizeof(T) == 2) {
+            const short8_t raw =
+                *reinterpret_cast<const short8_t*>(krow + ch * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) kv[un][i][e] = bf16_to_f32(raw[e]);
+          } else {
+            const float4_t raw =
+                *reinterpret_cast<const float4_t*>(krow + ch * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) kv[un][i][e] = raw[e];
+          }
+        }
+      }
+#pragma unroll
+      for (int un = 0; un < UNR; un++) {
+        const int kk = kb + 32 * un;
+        const float dist = (float)(pos - (lo + k0 + kk));
+#pragma unroll
+        for (int r = 0; r < RT; r++) {
+          float dot = 0.0f;       // q slices of missing chunks are zero
+#pragma unroll
+          for (int i = 0; i < NCH; i++)
+#pragma unroll
+            for (int e = 0; e < VEC; e++) dot += qreg[r][i][e] * kv[un][i][e];
+          float sv = group_reduce_sum<8>(dot) * scale;
+          if (softcap > 0.f) sv = softcap * tanhf(sv / softcap);
+          if (r1) sv -= hr1[r] * log1pf(hr2[r] * dist);
+          if (sub == 0 && r < nr && kk < nk) s_s[r * KT + kk] = sv;
+        }
+        if (sub == 0 && kk < nk) row_s[kk] = rowi[un];
+      }
+    }
+    __syncthreads();
+    // ---- softmax statistics of the tile, one head per wave at a time
+    for (int r = wave; r < nr; r += 4) {
+      float mx = -INFINITY;
+      for (int kk = lane; kk < nk; kk += 64) mx = fmaxf(mx, s_s[r * KT + kk]);
+      mx = wave_reduce_max(mx);
+      const float m_old = m_s[r];
+      const float m_new = fmaxf(m_old, mx);
+      float sum = 0.0f;
+      for (int kk = lane; kk < nk; kk += 64) {
+        const float p = expf(s_s[r * KT + kk] - m_new);
+        s_s[r * KT + kk] = p;
+        sum += p;
+      }
+      sum = wave_reduce_sum(sum);
+      if (lane == 0) {
+        const float corr = expf(m_old - m_new);      // 0 on the first tile
+        c_s[r] = corr;
+        l_s[r] = l_s[r] * corr + sum;
+        m_s[r] = m_new;
+      }
+    }
+    __syncthreads();
+    // ---- P.V
+#pragma unroll
+    for (int r = 0; r < RT; r++) {
+      const float corr = r < nr ? c_s[r] : 0.0f;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) acc[r][e] *= corr;
+    }
+    const int rows_trip = 4 * rpw;           // rows per un-step, all waves
+    for (int kb = wave * rpw + rsub; kb < nk; kb += rows_trip * UNR) {
+      float vv[UNR][VEC], pw[UNR][RT];
+#pragma unroll
+      for (int un = 0; un < UNR; un++) {
+        const int kk = min(kb + rows_trip * un, nk - 1);
+        const bool ok = vlive && kb + rows_trip * un < nk;
+        const T* vrow = v_cache + (int64_t)row_s[kk] * V +
+                        min(vch, vchunks - 1) * VEC;
+        if constexpr (sizeof(T) == 2) {
+          const short8_t raw = *reinterpret_cast<const short8_t*>(vrow);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) vv[un][e] = bf16_to_f32(raw[e]);
+        } else {
+          const float4_t raw = *reinterpret_cast<const float4_t*>(vrow);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) vv[un][e] = raw[e];
+        }
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+          pw[un][r] = (ok && r < nr) ? s_s[r * KT + kk] : 0.0f;
+      }
+#pragma unroll
+      for (int un = 0; un < UNR; un++)
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+#pragma unroll
+          for (int e = 0; e < VEC; e++) acc[r][e] += pw[un][r] * vv[un][e];
+    }
+  }
+  // ---- fold: row groups inside the wave, then the four waves
+#pragma unroll
+  for (int r = 0; r < RT; r++)
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      float a = acc[r][e];
+      for (int off = lpr; off < 64; off <<= 1) a += __shfl_xor(a, off, 64);
+      if (rsub == 0 && vlive)
+        acc_s[(wave * RT + r) * 256 + vch * VEC + e] = a;
+    }
+  __syncthreads();
+  for (int e = tid; e < nr * V; e += 256) {
+    const int r = e / V, j = e % V;
+    float a = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) a += acc_s[(w * RT + r) * 256 + j];
+    act_st(out + ((int64_t)t * H + h0 + r) * V + j, a / l_s[r]);
+  }
+}
+
+template <typename T, int RT>
+void launch_decode(int nch, dim3 grid, size_t lds_bytes, hipStream_t stream,
+                   at::Tensor& out, const at::Tensor& q,
+                   const at::Tensor& k_cache, const at::Tensor& v_cache,
+                   const at::Tensor& block_tables,
+                   const at::Tensor& token_seq, const at::Tensor& positions,
+                   float scale, float softcap, const float* r1,
+                   const float* r2, int window, int H, int G, int D, int V,
+                   int BS, int KT) {
+#define KAITO_WDEC(NCH_)                                                     \
+  if (nch == NCH_) {                                                         \
+    hipLaunchKernelGGL((window_attention_decode_kernel<T, RT, NCH_>), grid,  \
+        dim3(256), lds_bytes, stream, (T*)out.data_ptr(),                    \
+        (const T*)q.data_ptr(), (const T*)k_cache.data_ptr(),                \
+        (const T*)v_cache.data_ptr(), block_tables.data_ptr<int>(),          \
+        (int)block_tables.size(1), token_seq.data_ptr<int>(),                \
+        positions.data_ptr<int64_t>(), scale, softcap, r1, r2, window, H, G, \
+        D, V, BS, KT);                                                       \
+    return;                                                                  \
+  }
+  KAITO_WDEC(1) KAITO_WDEC(2) KAITO_WDEC(4)
+#undef KAITO_WDEC
+}
+
+// Whether the decode kernel takes these sizes (16-byte chunks of the key
+// and value rows, at most 32 chunks per key, value rows of at most 256).
+inline bool decode_kernel_fits(int D, int V, int elem) {
+  const int vec = 16 / elem;
+  return D % vec == 0 && D / vec <= 32 && V % vec == 0 && V <= 256;
+}
+
 }  // namespace
 
 void qk_norm_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor k,
@@ -455,6 +700,48 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
   }
   TORCH_CHECK((int64_t)k_cache.size(0) * G * BS < (1ll << 31));
   if (T == 0) return;
+  auto stream0 = at::hip::getCurrentHIPStream();
+  if (decode_kernel_fits(D, V, (int)q.element_size())) {
+    const int R = H / G;
+    // heads per workgroup: share K/V reads across the group when the step
+    // has rows enough to fill the chip, else favour more workgroups
+    int rt = R >= 8 ? 8 : (R > 2 ? 4 : (R == 2 ? 2 : 1));
+    while (rt > 1 && (int64_t)T * G * ((R + rt - 1) / rt) < 1024) rt >>= 1;
+    const int vec = 16 / (int)q.element_size();
+    const int chunks = D / vec;
+    const int nch = chunks <= 8 ? 1 : (chunks <= 16 ? 2 : 4);
+    int KT = rt == 8 ? 512 : 1024;         // keeps the LDS stage under 64 KB
+    if (window > 0 && window < KT) KT = ((int)window + 31) / 32 * 32;
+    const size_t lds_bytes =
+        ((size_t)rt * KT + KT + 3 * rt + 4 * rt * 256) * 4;
+    const dim3 grid(T, G, (R + rt - 1) / rt);
+    const float* p1 = bias ? r1.data_ptr<float>() : nullptr;
+    const float* p2 = bias ? r2.data_ptr<float>() : nullptr;
+    KAITO_DISPATCH_ACT(q, {
+      if (rt == 8)
+        launch_decode<act_t, 8>(nch, grid, lds_bytes, stream0, out, q,
+            k_cache, v_cache, block_tables, token_seq, positions,
+            (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
+            BS, KT);
+      else if (rt == 4)
+        launch_decode<act_t, 4>(nch, grid, lds_bytes, stream0, out, q,
+            k_cache, v_cache, block_tables, token_seq, positions,
+            (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
+            BS, KT);
+      else if (rt == 2)
+        launch_decode<act_t, 2>(nch, grid, lds_bytes, stream0, out, q,
+            k_cache, v_cache, block_tables, token_seq, positions,
+            (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
+            BS, KT);
+      else
+        launch_decode<act_t, 1>(nch, grid, lds_bytes, stream0, out, q,
+            k_cache, v_cache, block_tables, token_seq, positions,
+            (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
+            BS, KT);
+    });
+    return;
+  }
+  // other sizes: one head per workgroup, one key per thread
   // keys per tile: the window when it is short, else 256
   int threads = 256;
   if (window > 0 && window <= 64) threads = 64;

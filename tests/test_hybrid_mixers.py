@@ -240,7 +240,10 @@ def run_attention(dev, dt, q, k, v, runs, window, scale, cap, r1, r2,
                                             (2, 1, 24, 40, 1),
                                             (3, 3, 8, 24, 21),
                                             (2, 2, 64, 128, 40),
-                                            (2, 1, 16, 16, 0)])
+                                            (2, 1, 16, 16, 0),
+                                            (2, 1, 10, 12, 5),
+                                            (16, 1, 16, 8, 9),
+                                            (1, 1, 16, 320, 4)])
 def test_window_attention_matches_plain(mode, H, G, D, V, window):
     dev, dt = mode
     T = 45
