@@ -13,10 +13,12 @@
 //
 // Three launches:
 //   1. prep (token-parallel): unit-norm q/k, decay and beta → f32 scratch
-//   2. recurrence: one workgroup per (chunk, head); thread (j, part) owns
-//      rows [part*DP, part*DP+DP) of column j of S in registers; tokens are
-//      staged through LDS eight at a time, so the token loop itself has no
-//      barrier and the only cross-lane traffic is the PARTS-wide butterfly
+//   2. recurrence: thread (j, part) owns rows [part*DP, part*DP+DP) of
+//      column j of S in registers; tokens are staged through LDS eight at
+//      a time, so the token loop itself has no barrier and the only
+//      cross-lane traffic is the PARTS-wide butterfly. Fast path: one
+//      single-wave workgroup per (chunk, head, group of columns); other
+//      sizes: one workgroup per (chunk, head)
 //   3. epilogue (token-parallel): RMS norm, weight, silu gate, store
 // A chunk that starts at position 0 starts from S = 0 whatever its slot
 // held; slots < 0 are padding and skipped.
@@ -311,8 +313,8 @@ __global__ void delta_epilogue_kernel(
     T* __restrict__ out,                                   // [T, H*V]
     const float* __restrict__ o,                           // [T, H, V]
     const T* __restrict__ gate, const int64_t g_s0, const int64_t g_s1,
-    const float* __restrict__ norm_w, const int* __restrict__ token_ok,
-    const int H, const int V, const float eps) {
+    const float* __restrict__ norm_w, const int H, const int V,
+    const float eps) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* orow = o + ((int64_t)t * H + h) * V;
   float ss = 0.f;
@@ -396,7 +398,7 @@ void run_delta(hipStream_t stream, at::Tensor& out, const at::Tensor& q,
   hipLaunchKernelGGL((delta_epilogue_kernel<T>), dim3(T_, H), dim3(64), 0,
       stream, (T*)out.data_ptr(), o.data_ptr<float>(),
       (const T*)gate.data_ptr(), gate.stride(0), gate.stride(1),
-      norm_w.data_ptr<float>(), nullptr, H, V, norm_eps);
+      norm_w.data_ptr<float>(), H, V, norm_eps);
 }
 #undef KAITO_DELTA_CASE
 

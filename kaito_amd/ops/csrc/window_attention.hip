@@ -10,12 +10,16 @@
 // [blocks, G, block_size, D|V] in the activation dtype. Scores, softmax
 // weights and the output accumulation are f32.
 //
-// window_attention_kernel: one workgroup per (query row, head). Keys are
-// taken a tile of blockDim keys at a time: one thread scores one key
-// (vector loads of its cache row), the tile's weights go through LDS, and
-// the P·V product is thread-per-value-dim, so consecutive lanes read
-// consecutive cache elements. Tiles are folded with the running-max
-// (online softmax) recurrence, so any window length works.
+// Three kernels share these semantics:
+//   window_attention_mfma_kernel   bf16 prompt portions, 64-row query tiles
+//   window_attention_decode_kernel single rows (and f32 portions), the
+//                                  heads of a kv group in one pass
+//   window_attention_kernel        any sizes: one workgroup per (row, head),
+//                                  one thread scores one key, the tile's
+//                                  weights go through LDS, P.V is
+//                                  thread-per-value-dim
+// All fold key tiles with the running-max (online softmax) recurrence, so
+// any window length works.
 #include "mix_common.h"
 
 namespace kaito {
@@ -394,9 +398,12 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
 //            DPP butterflies finish the dot products.
 //   softmax: wave r mod 4 owns head r: tile max, exp, sum, running max and
 //            sum with the rescale factor of the earlier tiles.
-//   P.V    : a wave takes every 4th key for all heads, a lane a slice of
-//            the value row (coalesced row reads), weights broadcast from
-//            LDS; the four waves' partial sums meet in LDS at the end.
+//   P.V    : LPR lanes cover one value row in 16-byte chunks, so one wave
+//            load touches 64 / LPR rows and UNR of them are in flight;
+//            weights are broadcast from LDS; the row groups of a wave are
+//            folded by shuffles and the four waves meet in LDS at the end.
+// The loops are unrolled by hand because the kernel is bound by the number
+// of bytes in flight, not by arithmetic.
 template <typename T, int RT, int NCH>
 __global__ __launch_bounds__(256) void window_attention_decode_kernel(
     T* __restrict__ out, const T* __restrict__ q,

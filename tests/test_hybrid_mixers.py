@@ -49,9 +49,10 @@ def split_runs(total, cuts):
 @pytest.mark.parametrize("taps,cuts", [(4, [1, 2, 3, 9, 10, 12]), (2, [5]),
                                        (3, [2, 4]), (1, [3]),
                                        (5, list(range(1, 14)))])
-def test_short_conv_portions(mode, taps, cuts):
+@pytest.mark.parametrize("C", [37, 64])
+def test_short_conv_portions(mode, taps, cuts, C):
     dev, dt = mode
-    C, T = 37, 14
+    T = 14
     x = torch.randn(T, C).to(dt)
     w, b = torch.randn(C, taps), torch.randn(C)
     want = O.silu(O.short_conv(x.double(), w.double(), b.double()))
