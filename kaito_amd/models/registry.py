@@ -348,3 +348,24 @@ register(ModelConfig(
     sliding_window=32, sliding_window_pattern="interleaved:2",
     moe_act="swiglu_oai", moe_bias=True, moe_routing="topk_softmax",
     attention_bias=True))
+
+
+def _tiny_gurapel() -> ModelConfig:
+    """A small hybrid stack for tests and smoke runs (random weights)."""
+    from .hybrid_config import gurapel_model_config
+    moe = {"kind": "moe", "expert": {"ff": 128},
+           "router": {"experts": 4, "top": 2}}
+    delta = {"type": "delta", "mlp": moe, "mixer": {
+        "heads": 4, "kv_heads": 2, "dim": 32, "vdim": 64, "conv": 4}}
+    par = {"type": "parallel", "mlp": moe, "mixer": {
+        "left": {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 64,
+                 "mask": {"size": 48}, "scale": 0.125, "softcap": 20.0},
+        "right": {"width": 256, "blocks": 4, "conv": 4}}}
+    return gurapel_model_config({
+        "architecture": "Gurapel", "embedding": {"scale": 1.0},
+        "layers": [delta, par, par, delta], "max_positions": 512,
+        "norm": {"eps": 1e-5}, "vocab": 512, "width": 256},
+        name="tiny-gurapel-test")
+
+
+register(_tiny_gurapel())

@@ -23,6 +23,7 @@
 // A chunk that starts at position 0 starts from S = 0 whatever its slot
 // held; slots < 0 are padding and skipped.
 #include "mix_common.h"
+#include <cstdlib>
 
 namespace kaito {
 
@@ -33,6 +34,7 @@ constexpr int TOK_TILE = 8;
 template <typename T>
 __global__ void delta_prep_kernel(
     float* __restrict__ qn, float* __restrict__ kn,      // [T, G, D]
+    float* __restrict__ kq,                               // [T, G] = qn . kn
     float* __restrict__ decay, float* __restrict__ beta,  // [T, H]
     const T* __restrict__ q, const int64_t q_s0, const int64_t q_s1,
     const T* __restrict__ k, const int64_t k_s0, const int64_t k_s1,
@@ -46,14 +48,16 @@ __global__ void delta_prep_kernel(
   const int lane = threadIdx.x;
   const T* qr = q + (int64_t)t * q_s0 + (int64_t)g * q_s1;
   const T* kr = k + (int64_t)t * k_s0 + (int64_t)g * k_s1;
-  float sq = 0.f, sk = 0.f;
+  float sq = 0.f, sk = 0.f, sqk = 0.f;
   for (int d = lane; d < D; d += 64) {
     const float qv = act_ld(qr + d), kv = act_ld(kr + d);
     sq += qv * qv;
     sk += kv * kv;
+    sqk += qv * kv;
   }
   sq = wave_reduce_sum(sq);
   sk = wave_reduce_sum(sk);
+  sqk = wave_reduce_sum(sqk);
   const float iq = (1.0f / sqrtf(sq + qk_eps)) * (1.0f / sqrtf((float)D));
   const float ik = 1.0f / sqrtf(sk + qk_eps);
   float* qo = qn + ((int64_t)t * G + g) * D;
@@ -62,6 +66,7 @@ __global__ void delta_prep_kernel(
     qo[d] = act_ld(qr + d) * iq;
     ko[d] = act_ld(kr + d) * ik;
   }
+  if (lane == 0) kq[(int64_t)t * G + g] = sqk * iq * ik;
   if (g == 0) {
     for (int h = lane; h < H; h += 64) {
       const float av = act_ld(a + (int64_t)t * a_s0 + h);
@@ -178,6 +183,7 @@ template <typename T, int DP, int PARTS>
 __global__ __launch_bounds__(64) void delta_recurrence_wave_kernel(
     float* __restrict__ o,                                 // [T, H, V]
     const float* __restrict__ qn, const float* __restrict__ kn,
+    const float* __restrict__ kq,
     const T* __restrict__ v, const int64_t v_s0, const int64_t v_s1,
     const float* __restrict__ decay, const float* __restrict__ beta,
     float* __restrict__ state,                             // [slots, H, D, V]
@@ -187,7 +193,13 @@ __global__ __launch_bounds__(64) void delta_recurrence_wave_kernel(
   constexpr int TT = TOK_TILE;
   constexpr int VB = 64 / PARTS;
   constexpr int DPAD = DP * PARTS;
-  constexpr int ROW = 2 * DPAD + VB + 4;      // k | q | v | decay beta - -
+  // In LDS each part's DP-slice of a k or q row is followed by 4 floats of
+  // padding: lanes of different parts read their slices in the same
+  // instruction, and slices a multiple of 32 floats apart would all land in
+  // the same banks.
+  constexpr int DPS = DP + 4;
+  constexpr int KROW = PARTS * DPS;
+  constexpr int ROW = 2 * KROW + VB + 4;      // k | q | v | decay beta k.q -
   constexpr int KQ4 = TT * DPAD / 4 / 64;     // float4 loads per lane
   constexpr int VN = (TT * VB + 63) / 64;
   __shared__ __attribute__((aligned(16))) float lds[2][TT * ROW];
@@ -234,10 +246,11 @@ __global__ __launch_bounds__(64) void delta_recurrence_wave_kernel(
           ? act_ld(v + (int64_t)(t0 + tt) * v_s0 + (int64_t)h * v_s1 + c)
           : 0.f;
     }
-    if (tid < 2 * TT) {
-      const int tt = tid >> 1;
-      const float* src = (tid & 1) ? beta : decay;
-      rdb = tt < nt ? src[(int64_t)(t0 + tt) * H + h] : 0.f;
+    if (tid < 3 * TT) {
+      const int tt = tid / 3, which = tid % 3;
+      if (tt >= nt) rdb = 0.f;
+      else if (which == 2) rdb = kq[(int64_t)(t0 + tt) * G + g];
+      else rdb = (which ? beta : decay)[(int64_t)(t0 + tt) * H + h];
     }
   };
   auto park = [&](float* buf) {
@@ -245,15 +258,16 @@ __global__ __launch_bounds__(64) void delta_recurrence_wave_kernel(
     for (int i = 0; i < KQ4; i++) {
       const int e = tid + i * 64;
       const int tt = e / (DPAD / 4), d = (e % (DPAD / 4)) * 4;
-      *reinterpret_cast<float4_t*>(buf + tt * ROW + d) = rk[i];
-      *reinterpret_cast<float4_t*>(buf + tt * ROW + DPAD + d) = rq[i];
+      const int dd = (d / DP) * DPS + d % DP;
+      *reinterpret_cast<float4_t*>(buf + tt * ROW + dd) = rk[i];
+      *reinterpret_cast<float4_t*>(buf + tt * ROW + KROW + dd) = rq[i];
     }
 #pragma unroll
     for (int i = 0; i < VN; i++) {
       const int e = tid + i * 64;
-      if (e < TT * VB) buf[(e / VB) * ROW + 2 * DPAD + e % VB] = rv[i];
+      if (e < TT * VB) buf[(e / VB) * ROW + 2 * KROW + e % VB] = rv[i];
     }
-    if (tid < 2 * TT) buf[(tid >> 1) * ROW + 2 * DPAD + VB + (tid & 1)] = rdb;
+    if (tid < 3 * TT) buf[(tid / 3) * ROW + 2 * KROW + VB + tid % 3] = rdb;
   };
 
   fetch(r0);
@@ -266,32 +280,39 @@ __global__ __launch_bounds__(64) void delta_recurrence_wave_kernel(
     if (more) fetch(t0 + TT);
     const float* buf = lds[cur];
     for (int tt = 0; tt < nt; tt++) {
-      const float* lk = buf + tt * ROW + d0;
-      const float* lq = lk + DPAD;
-      const float dec = buf[tt * ROW + 2 * DPAD + VB];
-      const float bet = buf[tt * ROW + 2 * DPAD + VB + 1];
-      const float vj = buf[tt * ROW + 2 * DPAD + jl];
-      float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
-#pragma unroll
-      for (int i = 0; i < DP; i += 4) {
-        const float4_t k4 = *reinterpret_cast<const float4_t*>(lk + i);
-        S[i] *= dec; S[i + 1] *= dec; S[i + 2] *= dec; S[i + 3] *= dec;
-        p0 += S[i] * k4[0]; p1 += S[i + 1] * k4[1];
-        p2 += S[i + 2] * k4[2]; p3 += S[i + 3] * k4[3];
-      }
-      const float pred = group_reduce_sum<PARTS>((p0 + p1) + (p2 + p3));
-      const float u = bet * (vj - pred);
-      p0 = p1 = p2 = p3 = 0.f;
+      const float* lk = buf + tt * ROW + part * DPS;
+      const float* lq = lk + KROW;
+      const float dec = buf[tt * ROW + 2 * KROW + VB];
+      const float bet = buf[tt * ROW + 2 * KROW + VB + 1];
+      const float kqv = buf[tt * ROW + 2 * KROW + VB + 2];
+      const float vj = buf[tt * ROW + 2 * KROW + jl];
+      // Both read-outs are taken from the state BEFORE this token: with
+      // S' = dec S + k u^T,  S'^T q = dec S^T q + u (k.q), so one pass and
+      // one reduction stage give the prediction and the output, and the
+      // update pass that follows has nothing waiting on it.
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
 #pragma unroll
       for (int i = 0; i < DP; i += 4) {
         const float4_t k4 = *reinterpret_cast<const float4_t*>(lk + i);
         const float4_t q4 = *reinterpret_cast<const float4_t*>(lq + i);
-        S[i] += k4[0] * u; S[i + 1] += k4[1] * u;
-        S[i + 2] += k4[2] * u; S[i + 3] += k4[3] * u;
-        p0 += S[i] * q4[0]; p1 += S[i + 1] * q4[1];
-        p2 += S[i + 2] * q4[2]; p3 += S[i + 3] * q4[3];
+        a0 += S[i] * k4[0]; a1 += S[i + 1] * k4[1];
+        a2 += S[i + 2] * k4[2]; a3 += S[i + 3] * k4[3];
+        b0 += S[i] * q4[0]; b1 += S[i + 1] * q4[1];
+        b2 += S[i + 2] * q4[2]; b3 += S[i + 3] * q4[3];
       }
-      const float oj = group_reduce_sum<PARTS>((p0 + p1) + (p2 + p3));
+      const float sk = group_reduce_sum<PARTS>((a0 + a1) + (a2 + a3));
+      const float sq = group_reduce_sum<PARTS>((b0 + b1) + (b2 + b3));
+      const float u = bet * (vj - dec * sk);
+      const float oj = dec * sq + u * kqv;
+#pragma unroll
+      for (int i = 0; i < DP; i += 4) {
+        const float4_t k4 = *reinterpret_cast<const float4_t*>(lk + i);
+        S[i] = dec * S[i] + k4[0] * u;
+        S[i + 1] = dec * S[i + 1] + k4[1] * u;
+        S[i + 2] = dec * S[i + 2] + k4[2] * u;
+        S[i + 3] = dec * S[i + 3] + k4[3] * u;
+      }
       if (live && part == 0)
         o[((int64_t)(t0 + tt) * H + h) * V + j] = oj;
     }
@@ -357,15 +378,16 @@ void run_delta(hipStream_t stream, at::Tensor& out, const at::Tensor& q,
                const at::Tensor& dt_bias, const at::Tensor& norm_w,
                at::Tensor& state, const at::Tensor& cu_seqlens,
                const at::Tensor& state_slots, const at::Tensor& seq_starts,
-               at::Tensor& qn, at::Tensor& kn, at::Tensor& decay,
-               at::Tensor& beta, at::Tensor& o, int dp, int parts,
+               at::Tensor& qn, at::Tensor& kn, at::Tensor& kq,
+               at::Tensor& decay, at::Tensor& beta, at::Tensor& o, int dp,
+               int parts,
                int threads, size_t lds_bytes, float qk_eps, float norm_eps) {
   const int T_ = q.size(0), G = q.size(1), D = q.size(2);
   const int H = v.size(1), V = v.size(2);
   const int B = state_slots.size(0);
   hipLaunchKernelGGL((delta_prep_kernel<T>), dim3(T_, G), dim3(64), 0,
       stream, qn.data_ptr<float>(), kn.data_ptr<float>(),
-      decay.data_ptr<float>(), beta.data_ptr<float>(),
+      kq.data_ptr<float>(), decay.data_ptr<float>(), beta.data_ptr<float>(),
       (const T*)q.data_ptr(), q.stride(0), q.stride(1),
       (const T*)k.data_ptr(), k.stride(0), k.stride(1),
       (const T*)a.data_ptr(), a.stride(0), (const T*)b.data_ptr(),
@@ -374,21 +396,32 @@ void run_delta(hipStream_t stream, at::Tensor& out, const at::Tensor& q,
   int wparts = 1;
   while (wparts * 32 < D) wparts <<= 1;
   if (D % 4 == 0 && wparts <= 8) {
-    // fast path: single-wave workgroups over groups of 64 / PARTS columns
-#define KAITO_DELTA_WAVE(PARTS_)                                             \
-    if (wparts == PARTS_) {                                                  \
+    // fast path: single-wave workgroups over groups of 64 / PARTS columns.
+    // A wave64 VALU instruction occupies its SIMD for four cycles and the
+    // token loop is serial, so the kernel is bound by how many SIMDs have a
+    // wave: with few (chunk, head, column-group) triples, halve the rows per
+    // lane (DP 16) to double the waves.
+    int dpw = 32;
+    const int64_t waves32 = (int64_t)B * H * ((V * wparts + 63) / 64);
+    // KAITO_DELTA_ROWS_PER_LANE=16|32 pins the choice (A/B runs, tests)
+    const char* pin = getenv("KAITO_DELTA_ROWS_PER_LANE");
+    const int want = pin ? atoi(pin) : (waves32 < 4096 ? 16 : 32);
+    if (want == 16 && wparts * 2 <= 16) { dpw = 16; wparts *= 2; }
+#define KAITO_DELTA_WAVE(DP_, PARTS_)                                        \
+    if (dpw == DP_ && wparts == PARTS_) {                                    \
       constexpr int VB = 64 / PARTS_;                                        \
-      hipLaunchKernelGGL((delta_recurrence_wave_kernel<T, 32, PARTS_>),      \
+      hipLaunchKernelGGL((delta_recurrence_wave_kernel<T, DP_, PARTS_>),     \
           dim3(B, H, (V + VB - 1) / VB), dim3(64), 0, stream,                \
           o.data_ptr<float>(), qn.data_ptr<float>(), kn.data_ptr<float>(),   \
-          (const T*)v.data_ptr(), v.stride(0), v.stride(1),                  \
-          decay.data_ptr<float>(), beta.data_ptr<float>(),                   \
+          kq.data_ptr<float>(), (const T*)v.data_ptr(), v.stride(0),         \
+          v.stride(1), decay.data_ptr<float>(), beta.data_ptr<float>(),      \
           state.data_ptr<float>(), cu_seqlens.data_ptr<int>(),               \
           state_slots.data_ptr<int>(), seq_starts.data_ptr<int>(), G, D, H,  \
           V);                                                                \
     }
-    KAITO_DELTA_WAVE(1) KAITO_DELTA_WAVE(2) KAITO_DELTA_WAVE(4)
-    KAITO_DELTA_WAVE(8)
+    KAITO_DELTA_WAVE(32, 1) KAITO_DELTA_WAVE(32, 2) KAITO_DELTA_WAVE(32, 4)
+    KAITO_DELTA_WAVE(32, 8) KAITO_DELTA_WAVE(16, 2) KAITO_DELTA_WAVE(16, 4)
+    KAITO_DELTA_WAVE(16, 8) KAITO_DELTA_WAVE(16, 16)
 #undef KAITO_DELTA_WAVE
   } else {
     KAITO_DELTA_CASE(32, 1) KAITO_DELTA_CASE(32, 2) KAITO_DELTA_CASE(32, 4)
@@ -439,6 +472,7 @@ void gated_delta_rule(at::Tensor out, at::Tensor q, at::Tensor k,
   auto f32 = q.options().dtype(at::kFloat);
   at::Tensor qn = at::empty({T, G, D}, f32), kn = at::empty({T, G, D}, f32);
   at::Tensor decay = at::empty({T, H}, f32), beta = at::empty({T, H}, f32);
+  at::Tensor kq = at::empty({T, G}, f32);
   // rows of padding chunks are never written by the recurrence: zero so
   // the epilogue reads defined values
   at::Tensor o = at::zeros({T, H, V}, f32);
@@ -458,7 +492,7 @@ void gated_delta_rule(at::Tensor out, at::Tensor q, at::Tensor k,
 
   KAITO_DISPATCH_ACT(q, {
     run_delta<act_t>(stream, out, q, k, v, gate, a, b, a_log, dt_bias, norm_w,
-                     state, cu_seqlens, state_slots, seq_starts, qn, kn,
+                     state, cu_seqlens, state_slots, seq_starts, qn, kn, kq,
                      decay, beta, o, dp, parts, threads, lds_bytes,
                      (float)qk_eps, (float)norm_eps);
   });

@@ -283,3 +283,41 @@ def test_graph_replayed_decode_matches_eager(tmp_path_factory):
         b = graphed.generate(prompts, sp)
         for x, y in zip(a, b):
             assert x.output_token_ids == y.output_token_ids
+
+
+def test_catalog_resolves_checkpoint_folder(tmp_path_factory):
+    """The server's way in: an unknown model name plus a weights folder
+    whose config.json names the design."""
+    from kaito_amd.models import get_model_config, resolve_model_class
+    cfg, W, folder = checkpoint(tmp_path_factory, "b")
+    mc = get_model_config("some-hybrid-checkpoint", weights_path=folder)
+    assert mc.arch == "gurapel" and mc.runtime == "native"
+    assert len(mc.layer_specs) == len(cfg["layers"])
+    assert mc.layer_specs[1].delta.dim == 40
+    assert mc.layer_specs[2].attn.window == 37
+    assert mc.layer_specs[1].moe is None
+    assert resolve_model_class(mc).__name__ == "GurapelForCausalLM"
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_random_init_preset_generates(device):
+    """The registered tiny preset with random weights through the normal
+    engine entry point (no checkpoint): batched sampling requests."""
+    import dataclasses
+    from kaito_amd.engine import EngineConfig, LLMEngine, SamplingParams
+    from kaito_amd.models import get_model_config
+    from kaito_amd.parallel.state import init_parallel
+    init_parallel(1)
+    mc = get_model_config("tiny-gurapel-test")
+    if device == "cpu":
+        mc = dataclasses.replace(mc, dtype=torch.float32)
+    eng = LLMEngine(EngineConfig(model=mc, device=device, max_num_seqs=4,
+                                 max_model_len=256, num_gpu_blocks=64,
+                                 enforce_eager=True))
+    prompts = [list(range(3, 3 + n)) for n in (40, 7, 19, 64, 5)]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=9, temperature=0.8,
+                                                top_p=0.9, seed=1,
+                                                ignore_eos=True))
+    assert [len(o.output_token_ids) for o in outs] == [9] * 5
+    assert eng.state_pool.num_free == 4
+    assert eng.pool.num_free == eng.pool.num_blocks

@@ -93,8 +93,14 @@ def plain_delta(q, k, v, gate, a, b, a_log, dt_bias, norm_w, eps):
                                      (2, 4, 48, 40), (1, 1, 128, 64),
                                      (1, 2, 64, 130), (1, 2, 10, 12),
                                      (1, 1, 256, 20)])
-def test_delta_rule_portions(mode, G, H, D, V):
+@pytest.mark.parametrize("rows_per_lane", ["16", "32"])
+def test_delta_rule_portions(mode, G, H, D, V, rows_per_lane, monkeypatch):
+    # both register tilings of the single-wave kernel (the launcher picks by
+    # the number of waves otherwise)
+    monkeypatch.setenv("KAITO_DELTA_ROWS_PER_LANE", rows_per_lane)
     dev, dt = mode
+    if dev == "cpu" and rows_per_lane == "32":
+        pytest.skip("kernel tiling is a GPU matter")
     T = 29
     r = lambda *s: torch.randn(*s).to(dt)
     q, k, v, gate = r(T, G, D), r(T, G, D), r(T, H, V), r(T, H, V)
