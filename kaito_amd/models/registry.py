@@ -356,15 +356,15 @@ def _tiny_gurapel() -> ModelConfig:
     moe = {"kind": "moe", "expert": {"ff": 128},
            "router": {"experts": 4, "top": 2}}
     delta = {"type": "delta", "mlp": moe, "mixer": {
-        "heads": 4, "kv_heads": 2, "dim": 32, "vdim": 64, "conv": 4}}
+        "heads": 6, "kv_heads": 3, "dim": 32, "vdim": 48, "conv": 3}}
     par = {"type": "parallel", "mlp": moe, "mixer": {
-        "left": {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 64,
+        "left": {"heads": 6, "kv_heads": 2, "dim": 64, "vdim": 64,
                  "mask": {"size": 48}, "scale": 0.125, "softcap": 20.0},
-        "right": {"width": 256, "blocks": 4, "conv": 4}}}
+        "right": {"width": 384, "blocks": 4, "conv": 3}}}
     return gurapel_model_config({
         "architecture": "Gurapel", "embedding": {"scale": 1.0},
-        "layers": [delta, par, par, delta], "max_positions": 512,
-        "norm": {"eps": 1e-5}, "vocab": 512, "width": 256},
+        "layers": [par, delta, par, delta], "max_positions": 512,
+        "norm": {"eps": 1e-6}, "vocab": 768, "width": 320},
         name="tiny-gurapel-test")
 
 
