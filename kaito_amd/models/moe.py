@@ -204,7 +204,8 @@ class MoEMLP(nn.Module):
         """Per-expert torch GEMMs (CPU tests / odd shapes). Host sync on
         the segment sizes — never used on the GPU hot path."""
         off = offsets.tolist()
-        out = torch.zeros_like(x)
+        # f32 accumulation over a token's experts, like the fused path
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
         idx64 = sorted_tok.long()
         for le in range(self.e_local):
             e = self.e_base + le
@@ -226,6 +227,5 @@ class MoEMLP(nn.Module):
             y = torch.nn.functional.linear(
                 act, self.w_down[le],
                 self.b_down[le] if self.b_down is not None else None)
-            out.index_add_(0, rows,
-                           (y.float() * gates[s:t, None]).to(out.dtype))
-        return out
+            out.index_add_(0, rows, y.float() * gates[s:t, None])
+        return out.to(x.dtype)
