@@ -219,7 +219,8 @@ __global__ void window_attention_kernel(
 // B-fragments are contiguous. S = Q K^T and O += P V run on
 // v_mfma_f32_16x16x32_bf16; scaling, capping, the distance penalty, the
 // window/causal mask and the online softmax are f32 on the accumulator
-// fragments. Key and value sizes are separate template parameters.
+// fragments; the f32 weights enter the P.V product as a bf16 value +
+// remainder pair. Key and value sizes are separate template parameters.
 constexpr int WQ_TILE = 64;
 constexpr int WKV_TILE = 32;
 constexpr int WPAD = 40;
@@ -258,7 +259,10 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
 
   __shared__ short lds_k[WKV_TILE * D];
   __shared__ short lds_vt[DV * WPAD];
+  // softmax weights as a bf16 pair (value + remainder): two MFMAs per value
+  // tile keep ~16 mantissa bits of the f32 weight in the P.V product
   __shared__ short lds_p[4][16 * WPAD];
+  __shared__ short lds_pl[4][16 * WPAD];
 
   const int qrow = q0 + wave * 16 + lo;
   const int qtok = tok0 + (qrow < q_len ? qrow : q_len - 1);
@@ -356,21 +360,30 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
       lrow[r] += ps;
     }
     {
-      short* pl = lds_p[wave];
+      short* ph = lds_p[wave];
+      short* pl = lds_pl[wave];
 #pragma unroll
       for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-        for (int r = 0; r < 4; r++)
-          pl[(hi * 4 + r) * WPAD + kt * 16 + lo] = f32_to_bf16(p[kt][r]);
+        for (int r = 0; r < 4; r++) {
+          const short hi16 = f32_to_bf16(p[kt][r]);
+          const int at = (hi * 4 + r) * WPAD + kt * 16 + lo;
+          ph[at] = hi16;
+          pl[at] = f32_to_bf16(p[kt][r] - bf16_to_f32(hi16));
+        }
     }
     __builtin_amdgcn_s_waitcnt(0);
     const bf16x8 pfrag = *reinterpret_cast<const bf16x8*>(
         &lds_p[wave][lo * WPAD + hi * 8]);
+    const bf16x8 pfrag_lo = *reinterpret_cast<const bf16x8*>(
+        &lds_pl[wave][lo * WPAD + hi * 8]);
 #pragma unroll
     for (int dt = 0; dt < DT; dt++) {
       const bf16x8 vf = *reinterpret_cast<const bf16x8*>(
           &lds_vt[(dt * 16 + lo) * WPAD + hi * 8]);
       ofrag[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pfrag, vf,
+                                                          ofrag[dt], 0, 0, 0);
+      ofrag[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pfrag_lo, vf,
                                                           ofrag[dt], 0, 0, 0);
     }
     __syncthreads();
