@@ -321,3 +321,23 @@ def test_random_init_preset_generates(device):
     assert [len(o.output_token_ids) for o in outs] == [9] * 5
     assert eng.state_pool.num_free == 4
     assert eng.pool.num_free == eng.pool.num_blocks
+
+
+def test_preemption_recomputes_state(tmp_path_factory):
+    """A page pool too small for all running sequences: the scheduler
+    preempts by recompute, the victim's state slot goes back to the pool and
+    its re-prefill starts from the zero state at position 0. The tokens must
+    equal those of an engine that never preempts."""
+    from kaito_amd.engine import SamplingParams
+    cfg, W, folder = checkpoint(tmp_path_factory, "a")
+    mode = ("cpu", "float32")
+    prompts = [tokens(cfg, 30, 70 + i) for i in range(3)]
+    sp = SamplingParams(max_tokens=40, ignore_eos=True)
+    roomy = engine(folder, mode, max_tokens=1024)
+    tight = engine(folder, mode, max_tokens=176)      # 11 pages for 3 x 70
+    want = [o.output_token_ids for o in roomy.generate(prompts, sp)]
+    got = tight.generate(prompts, sp)
+    assert any(s.epoch > 0 for s in got), "the tight pool must preempt"
+    assert [o.output_token_ids for o in got] == want
+    assert tight.state_pool.num_free == 4
+    assert tight.pool.num_free == tight.pool.num_blocks
