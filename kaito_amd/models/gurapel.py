@@ -26,7 +26,7 @@ import torch.nn.functional as F
 
 from .. import ops
 from ..engine.config import ModelConfig
-from ..parallel.state import get_state
+from .hybrid_base import HybridStackBase, MixerLayerBase
 from .hybrid_config import LayerSpec, layer_moe_config
 from .mixers import BiasedWindowAttention, GatedDeltaMixer, RGLRUMixer
 from .moe import MoEMLP
@@ -37,7 +37,7 @@ def _vec(n):
                         requires_grad=False)
 
 
-class HybridLayer(nn.Module):
+class HybridLayer(MixerLayerBase):
     def __init__(self, cfg: ModelConfig, spec: LayerSpec):
         super().__init__()
         self.cfg, self.spec = cfg, spec
@@ -63,20 +63,6 @@ class HybridLayer(nn.Module):
         return [self.mixer] if self.spec.kind == "delta" else \
             [self.attn, self.rglru]
 
-    def alloc_cache(self, num_blocks, block_size, num_slots, device) -> Dict:
-        out: Dict[str, torch.Tensor] = {}
-        for m in self.mixers():
-            for k, t in m.alloc_cache(num_blocks, block_size, num_slots,
-                                      device).items():
-                out[type(m).__name__ + "." + k] = t
-        return out
-
-    @staticmethod
-    def _view(cache, m):
-        pre = type(m).__name__ + "."
-        return {k[len(pre):]: t for k, t in cache.items()
-                if k.startswith(pre)}
-
     def forward(self, x32, xa, positions, cache, meta):
         cfg = self.cfg
         eps, dt = cfg.rms_eps, cfg.dtype
@@ -95,19 +81,9 @@ class HybridLayer(nn.Module):
         return xa
 
 
-class GurapelForCausalLM(nn.Module):
-    # the runner hands these models state slots and the unified chunk
-    # metadata, and never the rotary-model prefill fast path
-    uses_state_slots = True
-
+class GurapelForCausalLM(HybridStackBase):
     def __init__(self, cfg: ModelConfig):
-        super().__init__()
-        st = get_state()
-        if st.tp_size != 1 or st.pp_size != 1:
-            raise NotImplementedError(
-                "hybrid stacks run one replica per GPU (tp = pp = 1)")
-        assert cfg.layer_specs, "hybrid model needs layer_specs"
-        self.cfg = cfg
+        super().__init__(cfg)
         self.embed_tokens = nn.Embedding(cfg.vocab_size, cfg.hidden_size,
                                          dtype=cfg.dtype)
         self.embed_tokens.weight.requires_grad_(False)
@@ -120,14 +96,8 @@ class GurapelForCausalLM(nn.Module):
         self.lm_head = nn.Parameter(
             torch.empty(cfg.vocab_size, cfg.hidden_size, dtype=cfg.dtype),
             requires_grad=False)
-        # optional observer of the residual stream after each layer
-        self.layer_hook = None
 
     # ---- engine interface -------------------------------------------------
-    @property
-    def num_local_layers(self) -> int:
-        return len(self.layers)
-
     def decode_graph_capturable(self) -> bool:
         """True when no decode-step op reads device data on the host: the
         MoE layers must take the fused grouped-GEMM path (bf16, 64-aligned
@@ -138,24 +108,6 @@ class GurapelForCausalLM(nn.Module):
                 and self.cfg.hidden_size % 64 == 0
                 and layer.mlp.ie_local % 64 == 0)
             for layer in self.layers)
-
-    def init_rope(self, device, max_pos: Optional[int] = None):
-        """No rotation in this design."""
-
-    def cache_bytes(self, block_size: int):
-        """(bytes per KV page, bytes per state slot) over all layers."""
-        page = slot = 0
-        for layer in self.layers:
-            for m in layer.mixers():
-                p, s = m.cache_bytes(block_size)
-                page += p
-                slot += s
-        return page, slot
-
-    def alloc_caches(self, num_blocks, block_size, num_slots,
-                     device) -> List[Dict]:
-        return [layer.alloc_cache(num_blocks, block_size, num_slots, device)
-                for layer in self.layers]
 
     def forward(self, input_ids, positions, kv_caches, meta,
                 hidden_in=None) -> torch.Tensor:
@@ -168,12 +120,6 @@ class GurapelForCausalLM(nn.Module):
             if self.layer_hook is not None:
                 self.layer_hook(i, x32)
         return x32
-
-    def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
-        """hidden: rows of the f32 residual stream → f32 logits."""
-        h = ops.rms_norm_cast(hidden.contiguous(), self.norm,
-                              self.cfg.rms_eps, self.cfg.dtype)
-        return F.linear(h, self.lm_head).float()
 
     # ---- weights ----------------------------------------------------------
     @torch.no_grad()

@@ -1,6 +1,6 @@
 """Per-layer specifications for hybrid stacks (recurrent + windowed
-attention layers mixed in one model) and the config.json reader of the
-Gurapel design.
+attention layers mixed in one model) and the config.json readers of the
+Gurapel and Pokulorn designs.
 
 A homogeneous model is described by the flat ModelConfig fields; a hybrid
 one additionally carries `layer_specs`, one LayerSpec per layer, each
@@ -65,14 +65,113 @@ class MoESpec:
 
 
 @dataclass(frozen=True)
+class RotarySpec:
+    """Rotation of the first `dims` dimensions of each q/k head, dimension
+    i paired with i + dims/2. With `factor` > 0 the frequencies are
+    interpolated by parts (wavelengths beyond `original`/`slow` turns are
+    divided by `factor`, those below `original`/`fast` turns kept, a
+    linear ramp between) and cos/sin are scaled by 0.1·ln(factor) + 1."""
+    dims: int
+    base: float
+    factor: float = 0.0          # 0 = plain rotation
+    original: float = 0.0
+    fast: float = 32.0
+    slow: float = 1.0
+
+    def frequencies(self):
+        """(per-pair angular frequencies as a float64 list, magnitude)."""
+        import math
+        half = self.dims // 2
+        freq = [self.base ** (-2.0 * i / self.dims) for i in range(half)]
+        if self.factor <= 0:
+            return freq, 1.0
+
+        def turn_dim(turns: float) -> float:
+            return self.dims * math.log(
+                self.original / (2 * math.pi * turns)) / (2 * math.log(self.base))
+        lo = max(math.floor(turn_dim(self.fast)), 0)
+        hi = min(math.ceil(turn_dim(self.slow)), self.dims - 1)
+        out = []
+        for i, f in enumerate(freq):
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            out.append(f / self.factor * ramp + f * (1.0 - ramp))
+        return out, 0.1 * math.log(self.factor) + 1.0
+
+
+@dataclass(frozen=True)
+class RotaryAttnSpec:
+    """Softmax attention over the paged cache with short causal
+    convolutions on q/k/v, per-head qk RMS norm (shared weight), partial
+    rotation, and a choice of: sliding window that also keeps the first
+    tokens, a per-head sink term in the softmax denominator, blending of
+    the values with those of the stack's first value-mixing layer, and a
+    sigmoid output gate."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    conv_taps: int = 0            # 0 = no convolution
+    rot: Optional[RotarySpec] = None
+    window: int = 0               # 0 = every earlier key
+    keep_first: int = 0           # with a window: keys j < keep_first stay
+    sink: bool = False
+    mix_values: bool = False
+    gate: bool = False
+    qk_norm: bool = True
+
+
+@dataclass(frozen=True)
+class MLSTMSpec:
+    """Matrix-memory recurrence with an exponential input gate and a
+    sigmoid forget gate kept in the log domain under a running maximum;
+    gate pre-activations are soft-capped by cap·tanh(·/cap)."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+    denom_floor: float = 1e-6     # added to the read-out's denominator
+
+
+@dataclass(frozen=True)
+class SSDSpec:
+    """Selective state space with a scalar decay per head and step
+    (state [N, vdim] per head), B/C shared by heads of a group, short
+    convolution on x/B/C, silu(z) gate and a grouped RMS norm."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    norm_groups: int
+    conv_taps: int
+
+
+@dataclass(frozen=True)
+class DenseFFSpec:
+    """Gated feed-forward: g = min(gate, limit), u = clamp(up, ±limit),
+    y = g·sigmoid(alpha·g)·(u + 1)."""
+    ff: int
+    limit: float
+    alpha: float = 1.702
+
+
+@dataclass(frozen=True)
 class LayerSpec:
-    # "delta": one DeltaRuleSpec; "parallel": WindowAttnSpec beside
-    # RGLRUSpec, outputs normed and averaged
+    # Gurapel — "delta": one DeltaRuleSpec; "parallel": WindowAttnSpec
+    # beside RGLRUSpec, outputs normed and averaged.
+    # Pokulorn — "mlstm": MLSTMSpec; "attention": RotaryAttnSpec;
+    # "parallel": RotaryAttnSpec beside SSDSpec, outputs summed with the
+    # weights `branch_scales`.
     kind: str
     delta: Optional[DeltaRuleSpec] = None
     attn: Optional[WindowAttnSpec] = None
     rglru: Optional[RGLRUSpec] = None
     moe: Optional[MoESpec] = None     # None = no feed-forward
+    mlstm: Optional[MLSTMSpec] = None
+    rattn: Optional[RotaryAttnSpec] = None
+    ssd: Optional[SSDSpec] = None
+    dense: Optional[DenseFFSpec] = None
+    branch_scales: Tuple[float, float] = (1.0, 1.0)
 
 
 def _moe_spec(m) -> Optional[MoESpec]:
@@ -155,3 +254,90 @@ def layer_moe_config(cfg: ModelConfig, moe: MoESpec) -> ModelConfig:
         moe_intermediate_size=ff, moe_routing="topk_softmax",
         moe_act="silu", moe_bias=False, n_shared_experts=0,
         moe_router_fp32=True)
+
+
+# ---- Pokulorn ---------------------------------------------------------------
+
+def _rotary_spec(r) -> Optional[RotarySpec]:
+    if not r:
+        return None
+    sc = r.get("scaling") or {}
+    return RotarySpec(
+        dims=int(r["dims"]), base=float(r["base"]),
+        factor=float(sc.get("factor", 0.0)),
+        original=float(sc.get("original", 0.0)),
+        fast=float(sc.get("fast", 32.0)), slow=float(sc.get("slow", 1.0)))
+
+
+def _rotary_attn_spec(mx: dict, sink: bool, gate: bool) -> RotaryAttnSpec:
+    mask = mx.get("mask") or {}
+    return RotaryAttnSpec(
+        heads=int(mx["heads"]), kv_heads=int(mx["kv_heads"]),
+        dim=int(mx["dim"]), vdim=int(mx["vdim"]), scale=float(mx["scale"]),
+        conv_taps=int(mx.get("conv", 0)), rot=_rotary_spec(mx.get("rot")),
+        window=int(mask.get("size", 0)),
+        keep_first=int(mask.get("keep_first", 0)),
+        sink=sink, mix_values=bool(mx.get("v_mix", False)), gate=gate)
+
+
+def _dense_spec(m) -> Optional[DenseFFSpec]:
+    if m is None:
+        return None
+    if m.get("kind", "dense") != "dense":
+        raise ValueError(f"unsupported feed-forward kind {m.get('kind')!r}")
+    return DenseFFSpec(ff=int(m["ff"]), limit=float(m["limit"]))
+
+
+def _pokulorn_layer(entry: dict) -> LayerSpec:
+    kind, mx = entry["type"], entry["mixer"]
+    dense = _dense_spec(entry.get("mlp"))
+    if kind == "mlstm":
+        return LayerSpec(kind, mlstm=MLSTMSpec(
+            heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx["vdim"]),
+            gate_cap=float(mx["gate_cap"])), dense=dense)
+    if kind == "attention":
+        return LayerSpec(kind, rattn=_rotary_attn_spec(mx, sink=True,
+                                                       gate=False),
+                         dense=dense)
+    if kind == "parallel":
+        rt = mx["right"]
+        return LayerSpec(
+            kind, rattn=_rotary_attn_spec(mx["left"], sink=False, gate=True),
+            ssd=SSDSpec(heads=int(rt["heads"]), vdim=int(rt["vdim"]),
+                        state=int(rt["state"]), groups=int(rt["groups"]),
+                        norm_groups=int(rt["norm_groups"]),
+                        conv_taps=int(rt["conv"])),
+            branch_scales=(float(mx["left_scale"]), float(mx["right_scale"])),
+            dense=dense)
+    raise ValueError(f"unknown layer type {kind!r}")
+
+
+def is_pokulorn_config(cfg: dict) -> bool:
+    return cfg.get("architecture") == "Pokulorn"
+
+
+# the design has no position table, so its length limit is the engine's
+POKULORN_DEFAULT_MAX_POSITION = 1 << 17
+
+
+def pokulorn_model_config(cfg: dict, name: str = "",
+                          dtype: torch.dtype = torch.bfloat16) -> ModelConfig:
+    """config.json of a Pokulorn checkpoint → ModelConfig (every size, the
+    layer order and every per-model constant come from the file)."""
+    specs: Tuple[LayerSpec, ...] = tuple(
+        _pokulorn_layer(e) for e in cfg["layers"])
+    width = int(cfg["width"])
+    attn = next((s.rattn for s in specs if s.rattn is not None), None)
+    ff = next((s.dense for s in specs if s.dense is not None), None)
+    return ModelConfig(
+        name=name or "pokulorn", arch="pokulorn", layer_specs=specs,
+        hidden_size=width, num_layers=len(specs),
+        num_heads=attn.heads if attn else 1,
+        num_kv_heads=attn.kv_heads if attn else 1,
+        head_dim=attn.dim if attn else width,
+        intermediate_size=ff.ff if ff else width,
+        vocab_size=int(cfg["vocab"]),
+        max_position=int(cfg.get("max_positions",
+                                 POKULORN_DEFAULT_MAX_POSITION)),
+        rms_eps=float(cfg["norm"]["eps"]),
+        residual_fp32=True, dtype=dtype)

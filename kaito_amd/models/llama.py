@@ -47,6 +47,9 @@ class AttnMetadata:
     # 64-row query tiles of the chunks (steps that hold prompt portions)
     tile_seq: Optional[torch.Tensor] = None      # [tiles] int32
     tile_qbase: Optional[torch.Tensor] = None    # [tiles] int32
+    # values one layer of a step leaves for later layers of the same step
+    # (the model's forward sets an empty dict)
+    layer_shared: Optional[dict] = None
 
 
 def build_cos_sin_cache(cfg: ModelConfig, device, max_pos: Optional[int] = None,

@@ -26,6 +26,8 @@ def load_safetensors_weights(model, path: str,
                              skip_projections: bool = False) -> None:
     if getattr(model.cfg, "arch", "llama") == "gurapel":
         return load_gurapel_weights(model, path)
+    if getattr(model.cfg, "arch", "llama") == "pokulorn":
+        return load_pokulorn_weights(model, path)
     from safetensors.torch import safe_open
 
     cfg = model.cfg
@@ -250,33 +252,49 @@ def load_safetensors_weights(model, path: str,
 
 # ---- hybrid stacks ------------------------------------------------------
 
-def load_gurapel_weights(model, path: str) -> None:
-    """Gurapel checkpoint (flat tensor names, `l<i>.` per layer, linear
-    weights [out, in]) → GurapelForCausalLM. Fuses the per-mixer input
-    projections, folds the one-plus norm weights and the recurrence's
-    decay constant, and widens every small per-channel tensor to f32."""
-    from safetensors.torch import safe_open
+class _FlatCheckpoint:
+    """All tensors of a folder's safetensors files by name, with
+    shape-checked copies into parameters and a record of what was read."""
 
-    tensors: Dict[str, torch.Tensor] = {}
-    for f in sorted(Path(path).glob("*.safetensors")):
-        with safe_open(str(f), framework="pt", device="cpu") as sf:
-            for k in sf.keys():
-                tensors[k] = sf.get_tensor(k)
-    if not tensors:
-        raise FileNotFoundError(f"no safetensors under {path}")
-    cfg = model.cfg
-    used = set()
+    def __init__(self, path: str):
+        from safetensors.torch import safe_open
+        self.tensors: Dict[str, torch.Tensor] = {}
+        for f in sorted(Path(path).glob("*.safetensors")):
+            with safe_open(str(f), framework="pt", device="cpu") as sf:
+                for k in sf.keys():
+                    self.tensors[k] = sf.get_tensor(k)
+        if not self.tensors:
+            raise FileNotFoundError(f"no safetensors under {path}")
+        self.used = set()
 
-    def get(name):
-        used.add(name)
-        return tensors[name]
+    def get(self, name):
+        self.used.add(name)
+        return self.tensors[name]
 
+    @staticmethod
     def put(param, value):
         if tuple(param.shape) != tuple(value.shape):
             raise ValueError(f"shape mismatch: parameter {tuple(param.shape)}"
                              f" vs checkpoint {tuple(value.shape)}")
         with torch.no_grad():
             param.copy_(value.to(param.dtype))
+
+    def warn_unused(self):
+        extra = set(self.tensors) - self.used
+        if extra:
+            import logging
+            logging.getLogger(__name__).warning(
+                "checkpoint tensors not used by the model: %s",
+                sorted(extra)[:8])
+
+
+def load_gurapel_weights(model, path: str) -> None:
+    """Gurapel checkpoint (flat tensor names, `l<i>.` per layer, linear
+    weights [out, in]) → GurapelForCausalLM. Fuses the per-mixer input
+    projections, folds the one-plus norm weights and the recurrence's
+    decay constant, and widens every small per-channel tensor to f32."""
+    ck = _FlatCheckpoint(path)
+    get, put = ck.get, ck.put
 
     def one_plus(name):
         return get(name).float() + 1.0
@@ -341,8 +359,75 @@ def load_gurapel_weights(model, path: str) -> None:
                     mlp.w_gate_up[e, ie:ie + ff].copy_(
                         u.to(mlp.w_gate_up.dtype))
                     mlp.w_down[e, :, :ff].copy_(d.to(mlp.w_down.dtype))
-    extra = set(tensors) - used
-    if extra:
-        import logging
-        logging.getLogger(__name__).warning(
-            "checkpoint tensors not used by the model: %s", sorted(extra)[:8])
+    ck.warn_unused()
+
+
+def load_pokulorn_weights(model, path: str) -> None:
+    """Pokulorn checkpoint (flat tensor names, `l<i>.` per layer, mixer
+    tensors under `.mix.`, feed-forward under `.mlp.`, linear weights
+    [out, in]) → PokulornForCausalLM. Fuses each mixer's input
+    projections, splits off the small projections that feed recurrences
+    (kept f32) and widens every per-channel tensor to f32."""
+    ck = _FlatCheckpoint(path)
+    get, put = ck.get, ck.put
+
+    def load_attention(a, ap, first_mixer):
+        s = a.spec
+        names = ("q", "k", "v") + (("g",) if s.gate else ())
+        put(a.qkv_proj, torch.cat([get(ap + n) for n in names], 0))
+        if s.conv_taps > 0:
+            put(a.conv_weight, torch.cat(
+                [get(ap + n + ".conv") for n in ("q", "k", "v")], 0).float())
+        if s.qk_norm:
+            put(a.q_norm, get(ap + "q.norm").float())
+            put(a.k_norm, get(ap + "k.norm").float())
+        if s.sink:
+            put(a.sinks, get(ap + "sink").float())
+        if s.mix_values:
+            lam = float(get(ap + "vmix").float())
+            a.v_lambda = 0.0 if first_mixer else lam
+        put(a.o_proj, get(ap + "o"))
+
+    put(model.embed_tokens.weight, get("embed"))
+    put(model.norm, get("final.norm").float())
+    put(model.lm_head, get("head"))
+    seen_mixing = False
+    for i, layer in enumerate(model.layers):
+        pre = f"l{i}."
+        spec = layer.spec
+        put(layer.norm1, get(pre + "norm1").float())
+        if spec.kind == "mlstm":
+            m, mp = layer.mixer, pre + "mix."
+            put(m.in_proj, torch.cat(
+                [get(mp + n) for n in ("q", "k", "v", "g")], 0))
+            put(m.gate_proj, torch.cat(
+                [get(mp + "i"), get(mp + "f")], 0).float())
+            put(m.gate_bias, torch.cat(
+                [get(mp + "i.b"), get(mp + "f.b")], 0).float())
+            put(m.out_norm, get(mp + "norm").float())
+            put(m.o_proj, get(mp + "o"))
+        elif spec.kind == "attention":
+            load_attention(layer.attn, pre + "mix.", not seen_mixing)
+            seen_mixing = seen_mixing or spec.rattn.mix_values
+        else:
+            load_attention(layer.attn, pre + "mix.left.", not seen_mixing)
+            seen_mixing = seen_mixing or spec.rattn.mix_values
+            r, rp = layer.ssd, pre + "mix.right."
+            w_in = get(rp + "in")
+            main = r.inner + r.conv_ch          # rows [z | x | B | C], then dt
+            put(r.in_proj, w_in[:main])
+            put(r.dt_proj, w_in[main:].float())
+            put(r.conv_weight, get(rp + "conv").float())
+            put(r.conv_bias, get(rp + "conv.b").float())
+            put(r.a_log, get(rp + "A_log").float())
+            put(r.dt_bias, get(rp + "dt_bias").float())
+            put(r.d_skip, get(rp + "D").float())
+            put(r.out_norm, get(rp + "norm").float())
+            put(r.o_proj, get(rp + "o"))
+        if layer.mlp is not None:
+            fp = pre + "mlp."
+            put(layer.norm2, get(pre + "norm2").float())
+            put(layer.mlp.gate_up, torch.cat(
+                [get(fp + "gate"), get(fp + "up")], 0))
+            put(layer.mlp.down, get(fp + "down"))
+    ck.warn_unused()

@@ -1,9 +1,12 @@
 """Token mixers for hybrid stacks: gated delta rule, real-gated linear
-recurrence, and softmax attention over a sliding window with a distance
-penalty. Each is a self-contained module parameterised by its spec
-(models/hybrid_config.py), so a design picks and combines them freely.
+recurrence, matrix-memory (mLSTM) recurrence, scalar-decay selective
+state space, and softmax attention over the paged cache in two flavours
+(distance penalty without rotation; convolutions + rotation + window
+with kept first tokens + sink). Each is a self-contained module
+parameterised by its spec (models/hybrid_config.py), so a design picks
+and combines them freely.
 
-All three follow the same calling convention:
+All follow the same calling convention:
 
     mixer(x, positions, cache, meta) -> y            x, y: [T, hidden]
 
@@ -27,7 +30,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
-from .hybrid_config import DeltaRuleSpec, RGLRUSpec, WindowAttnSpec
+from .hybrid_config import (DeltaRuleSpec, DenseFFSpec, MLSTMSpec, RGLRUSpec,
+                            RotaryAttnSpec, SSDSpec, WindowAttnSpec)
 
 
 def _p(*shape, dtype):
@@ -217,3 +221,236 @@ class BiasedWindowAttention(nn.Module):
                                  s.scale, s.softcap, self.r1, self.r2,
                                  s.window, tiles=tiles)
         return F.linear(o.reshape(T, -1), self.o_proj)
+
+
+class RotaryWindowAttention(nn.Module):
+    """Grouped-query softmax attention over the paged cache. q, k and v
+    pass a short causal convolution (its tail is per-sequence state), q
+    and k a per-head RMS norm and a rotation of their first `rot.dims`
+    dimensions; the mask is causal, optionally a sliding window that
+    also keeps the first `keep_first` tokens; a per-head sink may join
+    the softmax denominator; values may be blended with those of the
+    stack's first value-mixing layer before they are cached; the heads'
+    outputs may be gated by sigmoid of a fourth projection."""
+
+    def __init__(self, hidden: int, spec: RotaryAttnSpec, dtype,
+                 norm_eps: float):
+        super().__init__()
+        assert spec.heads % spec.kv_heads == 0
+        self.spec, self.dtype, self.norm_eps = spec, dtype, norm_eps
+        s = spec
+        self.q_size = s.heads * s.dim
+        self.k_size = s.kv_heads * s.dim
+        self.v_size = s.kv_heads * s.vdim
+        self.o_size = s.heads * s.vdim
+        self.conv_ch = self.q_size + self.k_size + self.v_size
+        # fused input projection, rows [q | k | v | gate]
+        self.qkv_proj = _p(self.conv_ch + (self.o_size if s.gate else 0),
+                           hidden, dtype=dtype)
+        self.conv_weight = _p(self.conv_ch, s.conv_taps, dtype=torch.float32) \
+            if s.conv_taps > 0 else None
+        if s.qk_norm:
+            self.q_norm = _p(s.dim, dtype=torch.float32)
+            self.k_norm = _p(s.dim, dtype=torch.float32)
+        else:
+            self.q_norm = self.k_norm = None
+        if s.rot is not None:
+            assert s.rot.dims % 2 == 0 and s.rot.dims <= s.dim
+            freq, self.rot_mag = s.rot.frequencies()
+            self.register_buffer("inv_freq", torch.tensor(
+                freq, dtype=torch.float64).float(), persistent=False)
+        else:
+            self.inv_freq, self.rot_mag = None, 1.0
+        self.sinks = _p(s.heads, dtype=torch.float32) if s.sink else None
+        # blend weight of the first value-mixing layer's values; the first
+        # such layer of a stack never reads it
+        self.v_lambda = 0.0
+        self.o_proj = _p(hidden, self.o_size, dtype=dtype)
+
+    def alloc_cache(self, num_blocks, block_size, num_slots, device) -> Dict:
+        s = self.spec
+        out = {
+            "k": torch.zeros(num_blocks, s.kv_heads, block_size, s.dim,
+                             dtype=self.dtype, device=device),
+            "v": torch.zeros(num_blocks, s.kv_heads, block_size, s.vdim,
+                             dtype=self.dtype, device=device),
+        }
+        if s.conv_taps > 0:
+            out["conv"] = torch.zeros(num_slots, max(s.conv_taps - 1, 1),
+                                      self.conv_ch, dtype=self.dtype,
+                                      device=device)
+        return out
+
+    def cache_bytes(self, block_size: int):
+        s = self.spec
+        esz = torch.empty(0, dtype=self.dtype).element_size()
+        slot = max(s.conv_taps - 1, 1) * self.conv_ch * esz \
+            if s.conv_taps > 0 else 0
+        return s.kv_heads * block_size * (s.dim + s.vdim) * esz, slot
+
+    def forward(self, x, positions, cache, meta):
+        s = self.spec
+        T = x.size(0)
+        p = F.linear(x, self.qkv_proj)
+        qkv = p[:, :self.conv_ch]
+        if s.conv_taps > 0:
+            qkv = ops.causal_conv_update(
+                qkv, self.conv_weight, None, cache["conv"], meta.cu_seqlens,
+                meta.state_slots, meta.seq_starts, meta.token_seq, act=0)
+        q = qkv[:, :self.q_size].unflatten(-1, (s.heads, s.dim))
+        k = qkv[:, self.q_size:self.q_size + self.k_size].unflatten(
+            -1, (s.kv_heads, s.dim))
+        v = qkv[:, self.q_size + self.k_size:].unflatten(
+            -1, (s.kv_heads, s.vdim))
+        v_first, lam = None, 0.0
+        if s.mix_values:
+            shared = meta.layer_shared
+            if "v_first" in shared:
+                v_first, lam = shared["v_first"], self.v_lambda
+            else:
+                shared["v_first"] = v
+        qn = ops.qk_norm_cache_write(
+            q, k, v, self.q_norm, self.k_norm, self.norm_eps, cache["k"],
+            cache["v"], meta.slot_mapping, positions=positions,
+            inv_freq=self.inv_freq, rot_mag=self.rot_mag, v_first=v_first,
+            v_lambda=lam)
+        tiles = None
+        if meta.tile_seq is not None:
+            tiles = (meta.tile_seq, meta.tile_qbase, meta.cu_seqlens,
+                     meta.seq_starts)
+        o = ops.window_attention(qn, cache["k"], cache["v"],
+                                 meta.block_tables, meta.token_seq, positions,
+                                 s.scale, window=s.window, tiles=tiles,
+                                 keep_first=s.keep_first, sinks=self.sinks)
+        o = o.reshape(T, self.o_size)
+        if s.gate:
+            o = ops.sigmoid_mul(o, p[:, self.conv_ch:])
+        return F.linear(o, self.o_proj)
+
+
+class MLSTMMixer(nn.Module):
+    """Matrix memory with exponential gating (mLSTM): per head a [dim,
+    vdim] memory C, a normaliser n and a running maximum m of the log
+    gates. The gate pre-activations come from an f32 projection (they
+    enter the recurrence); q/k/v and the output gate from the
+    activation-dtype projection."""
+
+    def __init__(self, hidden: int, spec: MLSTMSpec, dtype, norm_eps: float):
+        super().__init__()
+        self.spec, self.dtype, self.norm_eps = spec, dtype, norm_eps
+        s = spec
+        self.n_qk = s.heads * s.dim
+        self.n_v = s.heads * s.vdim
+        # fused input projection, rows [q | k | v | output gate]
+        self.in_proj = _p(2 * self.n_qk + 2 * self.n_v, hidden, dtype=dtype)
+        # rows [input gate | forget gate]
+        self.gate_proj = _p(2 * s.heads, hidden, dtype=torch.float32)
+        self.gate_bias = _p(2 * s.heads, dtype=torch.float32)
+        self.out_norm = _p(self.n_v, dtype=torch.float32)
+        self.o_proj = _p(hidden, self.n_v, dtype=dtype)
+
+    def alloc_cache(self, num_blocks, block_size, num_slots, device) -> Dict:
+        s = self.spec
+        f32 = dict(dtype=torch.float32, device=device)
+        return {"c": torch.zeros(num_slots, s.heads, s.dim, s.vdim, **f32),
+                "n": torch.zeros(num_slots, s.heads, s.dim, **f32),
+                "m": torch.zeros(num_slots, s.heads, **f32)}
+
+    def cache_bytes(self, block_size: int):
+        s = self.spec
+        return 0, s.heads * (s.dim * s.vdim + s.dim + 1) * 4
+
+    def forward(self, x, positions, cache, meta):
+        s = self.spec
+        p = F.linear(x, self.in_proj)
+        gates = F.linear(x.float(), self.gate_proj, self.gate_bias)
+        nq, nv = self.n_qk, self.n_v
+        q = p[:, :nq].unflatten(-1, (s.heads, s.dim))
+        k = p[:, nq:2 * nq].unflatten(-1, (s.heads, s.dim))
+        v = p[:, 2 * nq:2 * nq + nv].unflatten(-1, (s.heads, s.vdim))
+        g = p[:, 2 * nq + nv:].unflatten(-1, (s.heads, s.vdim))
+        o = ops.mlstm_scan(
+            q, k, v, g, gates[:, :s.heads], gates[:, s.heads:], self.out_norm,
+            cache["c"], cache["n"], cache["m"], meta.cu_seqlens,
+            meta.state_slots, meta.seq_starts, s.gate_cap, s.dim ** -0.5,
+            self.norm_eps, s.denom_floor)
+        return F.linear(o, self.o_proj)
+
+
+class SSDMixer(nn.Module):
+    """Selective state space with one scalar decay per head and step
+    (state-space duality form): x, B, C pass a short convolution with
+    bias and silu; per head S <- exp(-exp(A)·d)·S + d·B xᵀ with step size
+    d = softplus(dt + bias), y = Sᵀ C + D·x; y·silu(z) is RMS-normed in
+    equal parts and projected out. The step-size pre-activation comes
+    from an f32 projection."""
+
+    def __init__(self, hidden: int, spec: SSDSpec, dtype, norm_eps: float):
+        super().__init__()
+        assert spec.heads % spec.groups == 0
+        self.spec, self.dtype, self.norm_eps = spec, dtype, norm_eps
+        s = spec
+        self.inner = s.heads * s.vdim
+        assert self.inner % s.norm_groups == 0
+        self.n_bc = s.groups * s.state
+        self.conv_ch = self.inner + 2 * self.n_bc
+        # fused input projection, rows [z | x | B | C]
+        self.in_proj = _p(self.inner + self.conv_ch, hidden, dtype=dtype)
+        self.dt_proj = _p(s.heads, hidden, dtype=torch.float32)
+        self.conv_weight = _p(self.conv_ch, s.conv_taps, dtype=torch.float32)
+        self.conv_bias = _p(self.conv_ch, dtype=torch.float32)
+        self.a_log = _p(s.heads, dtype=torch.float32)
+        self.dt_bias = _p(s.heads, dtype=torch.float32)
+        self.d_skip = _p(s.heads, dtype=torch.float32)
+        self.out_norm = _p(self.inner, dtype=torch.float32)
+        self.o_proj = _p(hidden, self.inner, dtype=dtype)
+
+    def alloc_cache(self, num_blocks, block_size, num_slots, device) -> Dict:
+        s = self.spec
+        return {
+            "conv": torch.zeros(num_slots, max(s.conv_taps - 1, 1),
+                                self.conv_ch, dtype=self.dtype, device=device),
+            "ssm": torch.zeros(num_slots, s.heads, s.state, s.vdim,
+                               dtype=torch.float32, device=device),
+        }
+
+    def cache_bytes(self, block_size: int):
+        s = self.spec
+        esz = torch.empty(0, dtype=self.dtype).element_size()
+        return 0, (max(s.conv_taps - 1, 1) * self.conv_ch * esz
+                   + s.heads * s.state * s.vdim * 4)
+
+    def forward(self, x, positions, cache, meta):
+        s = self.spec
+        p = F.linear(x, self.in_proj)
+        dt = F.linear(x.float(), self.dt_proj)
+        xbc = ops.causal_conv_update(
+            p[:, self.inner:], self.conv_weight, self.conv_bias,
+            cache["conv"], meta.cu_seqlens, meta.state_slots,
+            meta.seq_starts, meta.token_seq, act=1)
+        xs = xbc[:, :self.inner].unflatten(-1, (s.heads, s.vdim))
+        B = xbc[:, self.inner:self.inner + self.n_bc].unflatten(
+            -1, (s.groups, s.state))
+        C = xbc[:, self.inner + self.n_bc:].unflatten(-1, (s.groups, s.state))
+        y = ops.ssd_scan(xs, B, C, dt, p[:, :self.inner], self.a_log,
+                         self.dt_bias, self.d_skip, self.out_norm,
+                         cache["ssm"], meta.cu_seqlens, meta.state_slots,
+                         meta.seq_starts, s.norm_groups, self.norm_eps)
+        return F.linear(y, self.o_proj)
+
+
+class ClampedGLU(nn.Module):
+    """Dense gated feed-forward with a clamped gate and a shifted linear
+    branch: down(g·sigmoid(alpha·g)·(u + 1)), g = min(gate, limit),
+    u = clamp(up, ±limit)."""
+
+    def __init__(self, hidden: int, spec: DenseFFSpec, dtype):
+        super().__init__()
+        self.spec = spec
+        self.gate_up = _p(2 * spec.ff, hidden, dtype=dtype)   # [gate | up]
+        self.down = _p(hidden, spec.ff, dtype=dtype)
+
+    def forward(self, x):
+        a = ops.clamped_glu(F.linear(x, self.gate_up), self.spec.limit,
+                            self.spec.alpha)
+        return F.linear(a, self.down)

@@ -24,6 +24,7 @@ def register(cfg: ModelConfig) -> ModelConfig:
 MODEL_CLASSES: Dict[str, str] = {
     "llama": "kaito_amd.models.llama:LlamaForCausalLM",
     "gurapel": "kaito_amd.models.gurapel:GurapelForCausalLM",
+    "pokulorn": "kaito_amd.models.pokulorn:PokulornForCausalLM",
 }
 
 
@@ -41,10 +42,13 @@ def config_from_checkpoint(cfg_json: dict, name: str = "",
                            dtype=None) -> ModelConfig:
     """config.json dict → ModelConfig, choosing the reader by the file's
     own architecture tag."""
-    from .hybrid_config import gurapel_model_config, is_gurapel_config
+    from .hybrid_config import (gurapel_model_config, is_gurapel_config,
+                                is_pokulorn_config, pokulorn_model_config)
+    kw = {"dtype": dtype} if dtype is not None else {}
     if is_gurapel_config(cfg_json):
-        kw = {"dtype": dtype} if dtype is not None else {}
         return gurapel_model_config(cfg_json, name=name, **kw)
+    if is_pokulorn_config(cfg_json):
+        return pokulorn_model_config(cfg_json, name=name, **kw)
     cfg = ModelConfig.from_hf_config(cfg_json, name=name)
     if dtype is not None:
         import dataclasses
@@ -369,3 +373,33 @@ def _tiny_gurapel() -> ModelConfig:
 
 
 register(_tiny_gurapel())
+
+
+def _tiny_pokulorn() -> ModelConfig:
+    """A small pre-norm hybrid stack (matrix memory, rotary window
+    attention with sinks and value mixing, attention beside a state-space
+    mixer) for tests and smoke runs (random weights)."""
+    from .hybrid_config import pokulorn_model_config
+    ff = {"kind": "dense", "ff": 192, "limit": 3.0}
+    rot = {"base": 10000.0, "dims": 16,
+           "scaling": {"factor": 8.0, "original": 256, "fast": 32.0,
+                       "slow": 1.0}}
+    mem = {"type": "mlstm", "mlp": None, "mixer": {
+        "heads": 2, "dim": 32, "vdim": 64, "gate_cap": 15.0}}
+    att = {"type": "attention", "mlp": ff, "mixer": {
+        "heads": 6, "kv_heads": 3, "dim": 32, "vdim": 16, "conv": 4,
+        "mask": {"size": 24, "keep_first": 4}, "rot": rot, "scale": 0.2,
+        "v_mix": True}}
+    par = {"type": "parallel", "mlp": ff, "mixer": {
+        "left": {"heads": 4, "kv_heads": 1, "dim": 32, "vdim": 32, "conv": 2,
+                 "rot": {"base": 5000.0, "dims": 32}, "scale": 0.18},
+        "right": {"heads": 6, "vdim": 16, "state": 24, "groups": 3,
+                  "norm_groups": 3, "conv": 3},
+        "left_scale": 0.7, "right_scale": 0.4}}
+    return pokulorn_model_config({
+        "architecture": "Pokulorn", "layers": [att, mem, par, att],
+        "norm": {"eps": 1e-5}, "vocab": 640, "width": 160,
+        "max_positions": 1024}, name="tiny-pokulorn-test")
+
+
+register(_tiny_pokulorn())

@@ -35,7 +35,8 @@ for _g, _names in {
     "mix": ("causal_conv_update gated_delta_rule rglru_scan "
             "qk_norm_cache_write window_attention window_attention_tiles "
             "post_norm_residual "
-            "rms_norm_cast"),
+            "rms_norm_cast mlstm_scan ssd_scan residual_add_norm "
+            "clamped_glu sigmoid_mul"),
 }.items():
     for _n in _names.split():
         _OP_GROUP[_n] = _g
@@ -431,29 +432,47 @@ def rglru_scan(u, gates, y, decay_rate, state, cu_seqlens, state_slots,
 
 
 def qk_norm_cache_write(q, k, v, q_w, k_w, eps: float, k_cache, v_cache,
-                        slot_mapping):
+                        slot_mapping, positions=None, inv_freq=None,
+                        rot_mag: float = 1.0, v_first=None,
+                        v_lambda: float = 0.0):
     """Per-head RMS norm of q [T, H, D] / k [T, G, D] (f32 weights [D] or
-    None) fused with the scatter of k and v [T, G, V] into the paged
-    caches [blocks, G, block_size, D|V]. Returns normed q [T, H, D]."""
+    None), optional rotation (inv_freq [R] f32: dim i of every head is
+    paired with dim i + R, angle = position * inv_freq[i] in f32, cos and
+    sin times rot_mag), optional value blend v <- (1 - v_lambda) v +
+    v_lambda v_first, fused with the scatter of k and v [T, G, V] into
+    the paged caches [blocks, G, block_size, D|V]. Returns q normed and
+    rotated, [T, H, D]."""
     if q.is_cuda:
         qn = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-        _K.qk_norm_cache_write(qn, q, k, v, _none(q_w, q), _none(k_w, q),
-                               eps, k_cache, v_cache, slot_mapping)
+        rot = inv_freq is not None and inv_freq.numel() > 0
+        _K.qk_norm_cache_write(
+            qn, q, k, v, _none(q_w, q), _none(k_w, q), eps, k_cache, v_cache,
+            slot_mapping,
+            positions if rot else torch.empty(0, dtype=torch.long,
+                                              device=q.device),
+            inv_freq if rot else _none(None, q), rot_mag,
+            v_first if v_first is not None else
+            torch.empty(0, dtype=q.dtype, device=q.device), v_lambda)
         return qn
     return torch_ref.qk_norm_cache_write(q, k, v, q_w, k_w, eps, k_cache,
-                                         v_cache, slot_mapping)
+                                         v_cache, slot_mapping, positions,
+                                         inv_freq, rot_mag, v_first, v_lambda)
 
 
-WINDOW_MFMA_SIZES = (64, 128, 256)
+WINDOW_MFMA_SIZES = (64, 128, 256)          # key sizes of the MFMA kernel
+WINDOW_MFMA_VSIZES = (32, 64, 128, 256)     # value sizes
 
 
 def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
                      scale: float, softcap: float = 0.0, r1=None, r2=None,
-                     window: int = 0, tiles=None):
-    """Causal sliding-window attention of query rows [T, H, D] over the
-    paged cache (key size D, value size V may differ), with optional tanh
-    score capping and the distance penalty r1*ln(1 + r2*distance).
-    Returns [T, H, V].
+                     window: int = 0, tiles=None, keep_first: int = 0,
+                     sinks=None):
+    """Causal attention of query rows [T, H, D] over the paged cache (key
+    size D, value size V may differ). A query at position i sees keys
+    j <= i with i - j < window or j < keep_first (window <= 0: all).
+    Options: tanh score capping, the distance penalty
+    r1*ln(1 + r2*distance), and per-head `sinks` [H] f32 whose exp joins
+    the softmax denominator. Returns [T, H, V].
 
     `tiles` = (tile_seq, tile_qbase, cu_seqlens, seq_starts) describes the
     step's chunks as 64-row query tiles (build_query_tiles); with it, bf16
@@ -466,20 +485,21 @@ def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
                           device=q.device)
         if (tiles is not None and q.dtype == torch.bfloat16
                 and D in WINDOW_MFMA_SIZES
-                and v_cache.size(3) in WINDOW_MFMA_SIZES):
+                and v_cache.size(3) in WINDOW_MFMA_VSIZES):
             tile_seq, tile_qbase, cu, starts = tiles
             _K.window_attention_tiles(
                 out, q, k_cache, v_cache, block_tables, tile_seq, tile_qbase,
                 cu, starts, scale, softcap, _none(r1, q), _none(r2, q),
-                window)
+                window, keep_first, _none(sinks, q))
             return out
         _K.window_attention(out, q, k_cache, v_cache, block_tables, token_seq,
                             positions, scale, softcap, _none(r1, q),
-                            _none(r2, q), window)
+                            _none(r2, q), window, keep_first,
+                            _none(sinks, q))
         return out
     return torch_ref.window_attention(q, k_cache, v_cache, block_tables,
                                       token_seq, positions, scale, softcap,
-                                      r1, r2, window)
+                                      r1, r2, window, keep_first, sinks)
 
 
 def build_query_tiles(chunk_lens, device):
@@ -517,3 +537,77 @@ def rms_norm_cast(x, weight, eps: float, out_dtype):
         _K.rms_norm_cast(out, x, weight, eps)
         return out
     return torch_ref.rms_norm_cast(x, weight, eps, out_dtype)
+
+
+def mlstm_scan(q, k, v, ogate, ipre, fpre, norm_w, state_c, state_n, state_m,
+               cu_seqlens, state_slots, seq_starts, cap: float,
+               q_scale: float, norm_eps: float, denom_floor: float = 1e-6):
+    """Matrix-memory (mLSTM) recurrence with fused gate activations,
+    normaliser, per-head RMS norm and sigmoid output gate. q/k [T, H, D],
+    v/ogate [T, H, V] (row strides free), ipre/fpre [T, H] f32; states
+    C [slots, H, D, V], n [slots, H, D], m [slots, H] f32 in place.
+    Returns [T, H*V]."""
+    if v.is_cuda:
+        T, H, V = v.shape
+        out = torch.empty(T, H * V, dtype=v.dtype, device=v.device)
+        _K.mlstm_scan(out, q, k, v, ogate, ipre, fpre, norm_w, state_c,
+                      state_n, state_m, cu_seqlens, state_slots, seq_starts,
+                      cap, q_scale, norm_eps, denom_floor)
+        return out
+    return torch_ref.mlstm_scan(q, k, v, ogate, ipre, fpre, norm_w, state_c,
+                                state_n, state_m, cu_seqlens, state_slots,
+                                seq_starts, cap, q_scale, norm_eps,
+                                denom_floor)
+
+
+def ssd_scan(x, B, C, dt, z, a_log, dt_bias, d_skip, norm_w, state,
+             cu_seqlens, state_slots, seq_starts, norm_groups: int,
+             norm_eps: float):
+    """Scalar-decay selective state space with fused step-size
+    activation, skip term, silu(z) gate and grouped RMS norm. x
+    [T, H, P], B/C [T, G, N], z [T, H*P] (row strides free), dt [T, H]
+    f32; state [slots, H, N, P] f32 in place. Returns [T, H*P]."""
+    if x.is_cuda:
+        T, H, P = x.shape
+        out = torch.empty(T, H * P, dtype=x.dtype, device=x.device)
+        _K.ssd_scan(out, x, B, C, dt, z, a_log, dt_bias, d_skip, norm_w,
+                    state, cu_seqlens, state_slots, seq_starts, norm_groups,
+                    norm_eps)
+        return out
+    return torch_ref.ssd_scan(x, B, C, dt, z, a_log, dt_bias, d_skip, norm_w,
+                              state, cu_seqlens, state_slots, seq_starts,
+                              norm_groups, norm_eps)
+
+
+def residual_add_norm(x32, y, w, eps: float, out_dtype, y2=None,
+                      s1: float = 1.0, s2: float = 1.0):
+    """Pre-norm residual step on an f32 stream [T, H]: x32 += s1*y
+    (+ s2*y2) in place; returns rms(x32)*w rounded to out_dtype, the next
+    sub-layer's input (None when w is None)."""
+    if x32.is_cuda:
+        h = torch.empty(x32.shape, dtype=out_dtype, device=x32.device) \
+            if w is not None else x32
+        _K.residual_add_norm(x32, h, y, _none(y2, y) if y2 is None else y2,
+                             _none(w, y), s1, s2, eps)
+        return h if w is not None else None
+    return torch_ref.residual_add_norm(x32, y, w, eps, out_dtype, y2, s1, s2)
+
+
+def clamped_glu(gu, limit: float, alpha: float = 1.702):
+    """[gate | up] rows [T, 2F] -> g*sigmoid(alpha*g)*(u + 1) [T, F] with
+    g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    if gu.is_cuda:
+        out = torch.empty(gu.size(0), gu.size(1) // 2, dtype=gu.dtype,
+                          device=gu.device)
+        _K.clamped_glu(out, gu, limit, alpha)
+        return out
+    return torch_ref.clamped_glu(gu, limit, alpha)
+
+
+def sigmoid_mul(x, gate):
+    """x [T, N] * sigmoid(gate [T, N]) (gate's row stride free)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _K.sigmoid_mul(out, x, gate)
+        return out
+    return torch_ref.sigmoid_mul(x, gate)

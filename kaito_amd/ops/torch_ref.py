@@ -346,17 +346,38 @@ def rglru_scan(u, gates, y, decay_rate, state, cu_seqlens, state_slots,
 
 
 def qk_norm_cache_write(q, k, v, q_w, k_w, eps: float, k_cache, v_cache,
-                        slot_mapping):
+                        slot_mapping, positions=None, inv_freq=None,
+                        rot_mag: float = 1.0, v_first=None,
+                        v_lambda: float = 0.0):
     """Per-head RMS norm of q [T, H, D] and k [T, G, D] (weights [D], or
-    None for no norm), then scatter k and v [T, G, V] into the paged
-    caches [blocks, G, block_size, D|V]. Returns the normed q."""
+    None for no norm), optional rotation of the first 2*len(inv_freq)
+    dims of every head (dim i paired with i + len(inv_freq); angle =
+    position * inv_freq[i]; cos and sin times rot_mag), optional blend
+    v <- (1 - v_lambda) v + v_lambda v_first, then scatter k and v
+    [T, G, V] into the paged caches [blocks, G, block_size, D|V].
+    Returns the normed (rotated) q."""
     def norm(t, w):
-        if w is None:
-            return t
         tf = t.float()
-        return (tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps)
-                * w.float()).to(t.dtype)
-    qn, kn = norm(q, q_w), norm(k, k_w)
+        if w is not None:
+            tf = tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps) \
+                * w.float()
+        return tf
+
+    def rot(tf):
+        if inv_freq is None or inv_freq.numel() == 0:
+            return tf
+        half = inv_freq.numel()
+        ang = positions.float()[:, None] * inv_freq.float()[None, :]
+        c = (torch.cos(ang) * rot_mag)[:, None, :]
+        s = (torch.sin(ang) * rot_mag)[:, None, :]
+        a, b = tf[..., :half], tf[..., half:2 * half]
+        return torch.cat([a * c - b * s, b * c + a * s, tf[..., 2 * half:]],
+                         -1)
+    qn = rot(norm(q, q_w)).to(q.dtype)
+    kn = rot(norm(k, k_w)).to(k.dtype)
+    if v_first is not None:
+        v = ((1.0 - v_lambda) * v.float() + v_lambda * v_first.float()) \
+            .to(v.dtype)
     bs = k_cache.size(2)
     for t, slot in enumerate(slot_mapping.tolist()):
         if slot < 0:
@@ -367,12 +388,14 @@ def qk_norm_cache_write(q, k, v, q_w, k_w, eps: float, k_cache, v_cache,
 
 
 def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
-                     scale: float, softcap: float, r1, r2, window: int):
+                     scale: float, softcap: float, r1, r2, window: int,
+                     keep_first: int = 0, sinks=None):
     """Causal sliding-window attention of query rows over the paged cache.
     Row t belongs to chunk token_seq[t] (its block table row) at sequence
-    position positions[t] and sees keys j with 0 <= pos - j < window
-    (window <= 0: all earlier keys). score = cap(q.k * scale) -
-    r1 * ln(1 + r2 * (pos - j))."""
+    position positions[t] and sees keys j <= pos with pos - j < window or
+    j < keep_first (window <= 0: all earlier keys). score =
+    cap(q.k * scale) - r1 * ln(1 + r2 * (pos - j)). With `sinks` [H] the
+    softmax denominator also holds exp(sink_h)."""
     T, H, D = q.shape
     G, bs, V = k_cache.size(1), k_cache.size(2), v_cache.size(3)
     rep = H // G
@@ -383,7 +406,8 @@ def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
             continue
         p = pos_l[t]
         lo = max(0, p - window + 1) if window > 0 else 0
-        js = torch.arange(lo, p + 1)
+        js = torch.cat([torch.arange(0, min(keep_first, lo)),
+                        torch.arange(lo, p + 1)])
         blk = block_tables[seq_l[t]].long()[js // bs]
         kk = k_cache[blk, :, js % bs].float()            # [n, G, D]
         vv = v_cache[blk, :, js % bs].float()
@@ -396,7 +420,12 @@ def window_attention(q, k_cache, v_cache, block_tables, token_seq, positions,
             dist = (p - js).float()
             s = s - r1.float()[:, None] * torch.log1p(
                 r2.float()[:, None] * dist[None, :])
-        out[t] = torch.einsum("hn,nhv->hv", torch.softmax(s, -1), vv)
+        if sinks is not None:
+            s = torch.cat([s, sinks.float()[:, None]], 1)
+            w = torch.softmax(s, -1)[:, :-1]
+        else:
+            w = torch.softmax(s, -1)
+        out[t] = torch.einsum("hn,nhv->hv", w, vv)
     return out.to(q.dtype)
 
 
@@ -421,3 +450,102 @@ def rms_norm_cast(x, weight, eps: float, out_dtype):
     xf = x.float()
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
             * weight.float()).to(out_dtype)
+
+
+def mlstm_scan(q, k, v, ogate, ipre, fpre, norm_w, state_c, state_n, state_m,
+               cu_seqlens, state_slots, seq_starts, cap: float,
+               q_scale: float, norm_eps: float, denom_floor: float):
+    """Matrix-memory recurrence. q/k [T, H, D], v/ogate [T, H, V], ipre /
+    fpre [T, H] f32 gate pre-activations; states C [slots, H, D, V],
+    n [slots, H, D], m [slots, H] f32, advanced in place. Log gates
+    i = cap*tanh(ipre/cap), f = logsigmoid(cap*tanh(fpre/cap)); running
+    maximum m (0 at the start of a sequence):
+        m' = max(f + m, i);  C' = e^(f+m-m') C + e^(i-m') k v^T  (n alike)
+        o  = C'^T q / (max(|n'.q|, e^(-m')) + denom_floor)
+    The read-out is RMS-normed per head, weighted, times sigmoid(ogate)."""
+    T, H, D = q.shape
+    V = v.shape[2]
+    qf, kf, vf = q.float() * q_scale, k.float(), v.float()
+    gi = cap * torch.tanh(ipre.float() / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(fpre.float() / cap))
+    o = torch.zeros(T, H, V)
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        if start > 0:
+            C, n, m = (state_c[slot].clone(), state_n[slot].clone(),
+                       state_m[slot].clone())
+        else:
+            C, n, m = torch.zeros(H, D, V), torch.zeros(H, D), torch.zeros(H)
+        for t in range(r0, r1):
+            m_new = torch.maximum(gf[t] + m, gi[t])
+            keep = torch.exp(gf[t] + m - m_new)
+            take = torch.exp(gi[t] - m_new)
+            C = keep[:, None, None] * C + take[:, None, None] * (
+                kf[t, :, :, None] * vf[t, :, None, :])
+            n = keep[:, None] * n + take[:, None] * kf[t]
+            m = m_new
+            den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) \
+                + denom_floor
+            o[t] = torch.einsum("hdv,hd->hv", C, qf[t]) / den[:, None]
+        state_c[slot], state_n[slot], state_m[slot] = C, n, m
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + norm_eps)
+    o = o.reshape(T, H * V) * norm_w.float() \
+        * torch.sigmoid(ogate.float().reshape(T, H * V))
+    return o.to(v.dtype)
+
+
+def ssd_scan(x, B, C, dt, z, a_log, dt_bias, d_skip, norm_w, state,
+             cu_seqlens, state_slots, seq_starts, norm_groups: int,
+             norm_eps: float):
+    """Selective state space with scalar decay. x [T, H, P], B/C
+    [T, G, N], dt [T, H] f32 (before bias and softplus), z [T, H*P];
+    state [slots, H, N, P] f32 in place. Per head (group h // (H/G)):
+        d = softplus(dt + dt_bias);  S' = e^(-e^(a_log) d) S + d B x^T
+        y = S'^T C + d_skip x
+    then y * silu(z), RMS norm in norm_groups equal parts, times norm_w."""
+    T, H, P = x.shape
+    G, N = B.shape[1], B.shape[2]
+    rep = H // G
+    xf = x.float()
+    Bf = B.float().repeat_interleave(rep, 1)
+    Cf = C.float().repeat_interleave(rep, 1)
+    d = torch.nn.functional.softplus(dt.float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * d)
+    y = torch.zeros(T, H, P)
+    for r0, r1, slot, start in _chunks(cu_seqlens, state_slots, seq_starts):
+        S = state[slot].clone() if start > 0 else torch.zeros(H, N, P)
+        for t in range(r0, r1):
+            S = decay[t, :, None, None] * S + d[t, :, None, None] * (
+                Bf[t, :, :, None] * xf[t, :, None, :])
+            y[t] = torch.einsum("hnp,hn->hp", S, Cf[t]) \
+                + d_skip.float()[:, None] * xf[t]
+        state[slot] = S
+    y = y.reshape(T, H * P) * torch.nn.functional.silu(z.float())
+    y = y.reshape(T, norm_groups, -1)
+    y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + norm_eps)
+    return (y.reshape(T, H * P) * norm_w.float()).to(x.dtype)
+
+
+def residual_add_norm(x32, y, w, eps: float, out_dtype, y2=None,
+                      s1: float = 1.0, s2: float = 1.0):
+    """Pre-norm residual step on an f32 stream: x32 += s1*y (+ s2*y2) in
+    place; returns rms(x32) * w rounded to out_dtype (None without w)."""
+    add = s1 * y.float() if s1 != 1.0 else y.float()
+    if y2 is not None:
+        add = add + s2 * y2.float()
+    x32 += add
+    if w is None:
+        return None
+    return rms_norm_cast(x32, w, eps, out_dtype)
+
+
+def clamped_glu(gu, limit: float, alpha: float):
+    """gu [T, 2F] = [gate | up] -> g*sigmoid(alpha*g)*(u + 1) with
+    g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    F_ = gu.size(-1) // 2
+    g = gu[..., :F_].float().clamp(max=limit)
+    u = gu[..., F_:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def sigmoid_mul(x, gate):
+    return (x.float() * torch.sigmoid(gate.float())).to(x.dtype)
