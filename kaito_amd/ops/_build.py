@@ -37,10 +37,12 @@ GROUPS: Dict[str, List[str]] = {
     "quant": ["bind_quant.cpp", "w4a16.hip", "lora.hip"],
     "comm": ["bind_comm.cpp", "allreduce_rmsnorm.hip"],
     # stateful sequence mixers of hybrid stacks: short convolutions, gated
-    # delta rule, gated linear recurrence, biased window attention, f32
-    # residual norms (each source registers its own ops)
+    # delta rule, gated linear recurrence, scalar-decay matrix recurrences
+    # (mLSTM, state-space duality), window attention, f32 residual norms,
+    # element-wise gates (each source registers its own ops)
     "mix": ["causal_conv.hip", "delta_rule.hip", "rglru.hip",
-            "window_attention.hip", "residual_norm.hip"],
+            "window_attention.hip", "residual_norm.hip",
+            "decay_recurrence.hip", "gated_act.hip"],
 }
 
 

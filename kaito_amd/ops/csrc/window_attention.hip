@@ -4,7 +4,15 @@
 //
 //   score(i, j) = cap * tanh(q_i . k_j * scale / cap)      (cap > 0)
 //                 - r1_h * ln(1 + r2_h * (i - j))           (r1 given)
-//   visible:      0 <= i - j < window   (window <= 0: every j <= i)
+//   visible:      j <= i and (i - j < window or j < keep_first)
+//                 (window <= 0: every j <= i)
+//   sinks:        with sink_h given, exp(sink_h) joins the softmax
+//                 denominator (no key, no value): the running maximum
+//                 starts at sink_h and the running sum at 1
+//
+// The q/k norm kernel optionally rotates the first 2R dims of every head
+// (dim i paired with i + R, angle = position * inv_freq[i], all f32) and
+// blends v with another layer's values before the cache write.
 //
 // Key size D and value size V are independent; caches are
 // [blocks, G, block_size, D|V] in the activation dtype. Scores, softmax
@@ -26,8 +34,37 @@ namespace kaito {
 
 namespace {
 
-// ---- q/k norm + cache scatter -------------------------------------------
+// ---- q/k norm (+ rotation) + cache scatter (+ value blend) ----------------
 // grid (T, H + 2G): blockIdx.y < H → q head; < H+G → k head; else v head.
+template <typename T>
+KAITO_DEV void norm_rotate_row(T* __restrict__ dst, const T* __restrict__ src,
+                               const float* __restrict__ w, const float eps,
+                               const int D, const float* __restrict__ inv_freq,
+                               const int R, const float pos,
+                               const float rot_mag, const int lane) {
+  float inv = 1.0f;
+  if (w != nullptr) {
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) { const float x = act_ld(src + d); ss += x * x; }
+    ss = wave_reduce_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)D + eps);
+  }
+  for (int d = lane; d < D; d += 64) {
+    float val;
+    if (d < 2 * R) {
+      const int i = d < R ? d : d - R;
+      const float a = act_ld(src + i) * inv * (w ? w[i] : 1.0f);
+      const float b = act_ld(src + i + R) * inv * (w ? w[i + R] : 1.0f);
+      const float ang = pos * inv_freq[i];
+      const float c = cosf(ang) * rot_mag, sn = sinf(ang) * rot_mag;
+      val = d < R ? a * c - b * sn : b * c + a * sn;
+    } else {
+      val = act_ld(src + d) * inv * (w ? w[d] : 1.0f);
+    }
+    act_st(dst + d, val);
+  }
+}
+
 template <typename T>
 __global__ void qk_norm_cache_write_kernel(
     T* __restrict__ q_out,                                   // [T, H, D]
@@ -37,20 +74,16 @@ __global__ void qk_norm_cache_write_kernel(
     const float* __restrict__ q_w, const float* __restrict__ k_w,
     const float eps, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const int64_t* __restrict__ slots, const int H, const int G, const int D,
-    const int V, const int BS) {
+    const int V, const int BS, const int64_t* __restrict__ positions,
+    const float* __restrict__ inv_freq, const int R, const float rot_mag,
+    const T* __restrict__ v_first, const int64_t vf_s0, const int64_t vf_s1,
+    const float v_lambda) {
   const int t = blockIdx.x, y = blockIdx.y, lane = threadIdx.x;
+  const float pos = R > 0 ? (float)positions[t] : 0.0f;
   if (y < H) {
-    const T* src = q + (int64_t)t * q_s0 + (int64_t)y * q_s1;
-    T* dst = q_out + ((int64_t)t * H + y) * D;
-    float inv = 1.0f;
-    if (q_w != nullptr) {
-      float ss = 0.f;
-      for (int d = lane; d < D; d += 64) { const float x = act_ld(src + d); ss += x * x; }
-      ss = wave_reduce_sum(ss);
-      inv = 1.0f / sqrtf(ss / (float)D + eps);
-    }
-    for (int d = lane; d < D; d += 64)
-      act_st(dst + d, act_ld(src + d) * inv * (q_w ? q_w[d] : 1.0f));
+    norm_rotate_row(q_out + ((int64_t)t * H + y) * D,
+                    q + (int64_t)t * q_s0 + (int64_t)y * q_s1, q_w, eps, D,
+                    inv_freq, R, pos, rot_mag, lane);
     return;
   }
   const int64_t slot = slots[t];
@@ -59,22 +92,21 @@ __global__ void qk_norm_cache_write_kernel(
   const int off = (int)(slot % BS);
   if (y < H + G) {
     const int g = y - H;
-    const T* src = k + (int64_t)t * k_s0 + (int64_t)g * k_s1;
-    T* dst = k_cache + ((blk * G + g) * BS + off) * D;
-    float inv = 1.0f;
-    if (k_w != nullptr) {
-      float ss = 0.f;
-      for (int d = lane; d < D; d += 64) { const float x = act_ld(src + d); ss += x * x; }
-      ss = wave_reduce_sum(ss);
-      inv = 1.0f / sqrtf(ss / (float)D + eps);
-    }
-    for (int d = lane; d < D; d += 64)
-      act_st(dst + d, act_ld(src + d) * inv * (k_w ? k_w[d] : 1.0f));
+    norm_rotate_row(k_cache + ((blk * G + g) * BS + off) * D,
+                    k + (int64_t)t * k_s0 + (int64_t)g * k_s1, k_w, eps, D,
+                    inv_freq, R, pos, rot_mag, lane);
   } else {
     const int g = y - H - G;
     const T* src = v + (int64_t)t * v_s0 + (int64_t)g * v_s1;
     T* dst = v_cache + ((blk * G + g) * BS + off) * V;
-    for (int d = lane; d < V; d += 64) dst[d] = src[d];
+    if (v_first != nullptr) {
+      const T* vf = v_first + (int64_t)t * vf_s0 + (int64_t)g * vf_s1;
+      for (int d = lane; d < V; d += 64)
+        act_st(dst + d, (1.0f - v_lambda) * act_ld(src + d) +
+                            v_lambda * act_ld(vf + d));
+    } else {
+      for (int d = lane; d < V; d += 64) dst[d] = src[d];
+    }
   }
 }
 
@@ -125,7 +157,8 @@ __global__ void window_attention_kernel(
     const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
     const float scale, const float softcap, const float* __restrict__ r1,
     const float* __restrict__ r2, const int window, const int H, const int G,
-    const int D, const int V, const int BS) {
+    const int D, const int V, const int BS, const int keep_first,
+    const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   const int KT = blockDim.x;            // keys per tile
   float* q_s = lds;                     // [D]
@@ -144,7 +177,8 @@ __global__ void window_attention_kernel(
   const int g = h / (H / G);
   const int pos = (int)positions[t];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int nkeys = pos - lo + 1;
+  const int nfirst = min(keep_first, lo);       // kept keys before the window
+  const int nkeys = nfirst + pos - lo + 1;
   const int* bt = block_tables + (int64_t)b * max_blocks;
   const float hr1 = r1 ? r1[h] : 0.0f, hr2 = r1 ? r2[h] : 0.0f;
 
@@ -156,14 +190,15 @@ __global__ void window_attention_kernel(
   float acc[MAXV];
 #pragma unroll
   for (int i = 0; i < MAXV; i++) acc[i] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = sinks ? sinks[h] : -INFINITY, l_run = sinks ? 1.0f : 0.f;
 
   for (int k0 = 0; k0 < nkeys; k0 += KT) {
     const int nk = min(KT, nkeys - k0);
     __syncthreads();                    // q_s ready / previous tile consumed
     float s = -INFINITY;
     if (tid < nk) {
-      const int j = lo + k0 + tid;
+      const int kx = k0 + tid;
+      const int j = kx < nfirst ? kx : lo + (kx - nfirst);
       const int page = bt[j / BS];
       const int64_t rowi = ((int64_t)page * G + g) * BS + (j % BS);
       blk_s[tid] = (int)rowi;
@@ -236,7 +271,7 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
     const int* __restrict__ block_tables, const int max_blocks,
     const float scale, const float softcap, const float* __restrict__ r1,
     const float* __restrict__ r2, const int window, const int H, const int G,
-    const int BS) {
+    const int BS, const int keep_first, const float* __restrict__ sinks) {
   constexpr int KK = D / 32;
   constexpr int DT = DV / 16;
   const int tile = blockIdx.x;
@@ -275,14 +310,21 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
   float mrow[4], lrow[4];
   f32x4 ofrag[DT];
 #pragma unroll
-  for (int r = 0; r < 4; r++) { mrow[r] = -1e30f; lrow[r] = 0.f; }
+  for (int r = 0; r < 4; r++) {
+    mrow[r] = sinks ? sinks[h] : -1e30f;
+    lrow[r] = sinks ? 1.0f : 0.f;
+  }
 #pragma unroll
   for (int dt = 0; dt < DT; dt++) ofrag[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int kv_end = min(kv_len, q_abs0 + q0 + WQ_TILE);
   const int kv_begin = (window > 0 && q_abs0 + q0 - window + 1 > 0)
       ? ((q_abs0 + q0 - window + 1) / WKV_TILE) * WKV_TILE : 0;
-  for (int kv0 = kv_begin; kv0 < kv_end; kv0 += WKV_TILE) {
+  // key tiles: those that hold kept first tokens, then the window's
+  const int first_end =
+      min((keep_first + WKV_TILE - 1) / WKV_TILE * WKV_TILE, kv_begin);
+  for (int kv0 = first_end > 0 ? 0 : kv_begin; kv0 < kv_end;
+       kv0 = (kv0 + WKV_TILE == first_end) ? kv_begin : kv0 + WKV_TILE) {
     for (int i = threadIdx.x; i < WKV_TILE * D / 8; i += 256) {
       const int row = (i * 8) / D;
       const int col = (i * 8) % D;
@@ -334,7 +376,7 @@ __global__ __launch_bounds__(256, 2) void window_attention_mfma_kernel(
         const int dist = q_abs - kvp;
         if (r1) sv -= hr1 * __logf(1.0f + hr2 * (float)max(dist, 0));
         if (dist < 0 || kvp >= kv_len || qr >= q_len ||
-            (window > 0 && dist >= window)) sv = -1e30f;
+            (window > 0 && dist >= window && kvp >= keep_first)) sv = -1e30f;
         p[kt][r] = sv;
       }
 #pragma unroll
@@ -425,7 +467,8 @@ __global__ __launch_bounds__(256) void window_attention_decode_kernel(
     const int* __restrict__ token_seq, const int64_t* __restrict__ positions,
     const float scale, const float softcap, const float* __restrict__ r1,
     const float* __restrict__ r2, const int window, const int H, const int G,
-    const int D, const int V, const int BS, const int KT) {
+    const int D, const int V, const int BS, const int KT,
+    const int keep_first, const float* __restrict__ sinks) {
   constexpr int VEC = 16 / (int)sizeof(T);
   extern __shared__ float lds[];
   float* s_s = lds;                            // [RT][KT]
@@ -451,7 +494,8 @@ __global__ __launch_bounds__(256) void window_attention_decode_kernel(
   }
   const int pos = (int)positions[t];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int nkeys = pos - lo + 1;
+  const int nfirst = min(keep_first, lo);       // kept keys before the window
+  const int nkeys = nfirst + pos - lo + 1;
   const int* bt = block_tables + (int64_t)b * max_blocks;
   const int nchunks = D / VEC;
 
@@ -485,7 +529,11 @@ __global__ __launch_bounds__(256) void window_attention_decode_kernel(
   for (int r = 0; r < RT; r++)
 #pragma unroll
     for (int e = 0; e < VEC; e++) acc[r][e] = 0.0f;
-  if (tid < RT) { m_s[tid] = -INFINITY; l_s[tid] = 0.0f; }
+  if (tid < RT) {
+    const bool sk = sinks != nullptr && tid < nr;
+    m_s[tid] = sk ? sinks[h0 + tid] : -INFINITY;
+    l_s[tid] = sk ? 1.0f : 0.0f;
+  }
 
   for (int k0 = 0; k0 < nkeys; k0 += KT) {
     const int nk = min(KT, nkeys - k0);
@@ -497,7 +545,8 @@ __global__ __launch_bounds__(256) void window_attention_decode_kernel(
       float kv[UNR][NCH][VEC];
 #pragma unroll
       for (int un = 0; un < UNR; un++) {
-        const int j = lo + k0 + min(kb + 32 * un, nk - 1);
+        const int kx = k0 + min(kb + 32 * un, nk - 1);
+        const int j = kx < nfirst ? kx : lo + (kx - nfirst);
         rowi[un] = (bt[j / BS] * G + g) * BS + (j % BS);
       }
 #pragma unroll
@@ -522,7 +571,9 @@ __global__ __launch_bounds__(256) void window_attention_decode_kernel(
 #pragma unroll
       for (int un = 0; un < UNR; un++) {
         const int kk = kb + 32 * un;
-        const float dist = (float)(pos - (lo + k0 + kk));
+        const int kx = k0 + kk;
+        const float dist =
+            (float)(pos - (kx < nfirst ? kx : lo + (kx - nfirst)));
 #pragma unroll
         for (int r = 0; r < RT; r++) {
           float dot = 0.0f;       // q slices of missing chunks are zero
@@ -626,7 +677,7 @@ void launch_decode(int nch, dim3 grid, size_t lds_bytes, hipStream_t stream,
                    const at::Tensor& token_seq, const at::Tensor& positions,
                    float scale, float softcap, const float* r1,
                    const float* r2, int window, int H, int G, int D, int V,
-                   int BS, int KT) {
+                   int BS, int KT, int keep_first, const float* sinks) {
 #define KAITO_WDEC(NCH_)                                                     \
   if (nch == NCH_) {                                                         \
     hipLaunchKernelGGL((window_attention_decode_kernel<T, RT, NCH_>), grid,  \
@@ -635,7 +686,7 @@ void launch_decode(int nch, dim3 grid, size_t lds_bytes, hipStream_t stream,
         (const T*)v_cache.data_ptr(), block_tables.data_ptr<int>(),          \
         (int)block_tables.size(1), token_seq.data_ptr<int>(),                \
         positions.data_ptr<int64_t>(), scale, softcap, r1, r2, window, H, G, \
-        D, V, BS, KT);                                                       \
+        D, V, BS, KT, keep_first, sinks);                                    \
     return;                                                                  \
   }
   KAITO_WDEC(1) KAITO_WDEC(2) KAITO_WDEC(4)
@@ -654,7 +705,9 @@ inline bool decode_kernel_fits(int D, int V, int elem) {
 void qk_norm_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor k,
                          at::Tensor v, at::Tensor q_w, at::Tensor k_w,
                          double eps, at::Tensor k_cache, at::Tensor v_cache,
-                         at::Tensor slot_mapping) {
+                         at::Tensor slot_mapping, at::Tensor positions,
+                         at::Tensor inv_freq, double rot_mag,
+                         at::Tensor v_first, double v_lambda) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && k.dim() == 3 && v.dim() == 3);
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   const int G = k.size(1), V = v.size(2);
@@ -677,6 +730,17 @@ void qk_norm_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor k,
   if (kn) { KAITO_CHECK_F32(k_w); TORCH_CHECK(k_w.numel() == D); }
   TORCH_CHECK(slot_mapping.is_cuda() && slot_mapping.dtype() == at::kLong &&
               slot_mapping.is_contiguous() && slot_mapping.size(0) == T);
+  const int R = (int)inv_freq.numel();
+  if (R > 0) {
+    KAITO_CHECK_F32(inv_freq);
+    TORCH_CHECK(2 * R <= D, "rotated dims exceed the head size");
+    TORCH_CHECK(positions.is_cuda() && positions.dtype() == at::kLong &&
+                positions.is_contiguous() && positions.size(0) == T);
+  }
+  const bool blend = v_first.numel() > 0;
+  if (blend)
+    TORCH_CHECK(v_first.dim() == 3 && v_first.sizes() == v.sizes() &&
+                v_first.stride(2) == 1 && v_first.dtype() == v.dtype());
   if (T == 0) return;
   auto stream = at::hip::getCurrentHIPStream();
   KAITO_DISPATCH_ACT(q, {
@@ -688,7 +752,12 @@ void qk_norm_cache_write(at::Tensor q_out, at::Tensor q, at::Tensor k,
         qn ? q_w.data_ptr<float>() : nullptr,
         kn ? k_w.data_ptr<float>() : nullptr, (float)eps,
         (act_t*)k_cache.data_ptr(), (act_t*)v_cache.data_ptr(),
-        slot_mapping.data_ptr<int64_t>(), H, G, D, V, BS);
+        slot_mapping.data_ptr<int64_t>(), H, G, D, V, BS,
+        R > 0 ? positions.data_ptr<int64_t>() : nullptr,
+        R > 0 ? inv_freq.data_ptr<float>() : nullptr, R, (float)rot_mag,
+        blend ? (const act_t*)v_first.data_ptr() : nullptr,
+        blend ? v_first.stride(0) : 0, blend ? v_first.stride(1) : 0,
+        (float)v_lambda);
   });
 }
 
@@ -696,9 +765,17 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                       at::Tensor v_cache, at::Tensor block_tables,
                       at::Tensor token_seq, at::Tensor positions,
                       double scale, double softcap, at::Tensor r1,
-                      at::Tensor r2, int64_t window) {
+                      at::Tensor r2, int64_t window, int64_t keep_first,
+                      at::Tensor sinks) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() &&
               is_act_dtype(q));
+  TORCH_CHECK(keep_first >= 0 && keep_first < (1 << 30));
+  const int kf = window > 0 ? (int)keep_first : 0;
+  const bool has_sinks = sinks.numel() > 0;
+  if (has_sinks) {
+    KAITO_CHECK_F32(sinks);
+    TORCH_CHECK(sinks.numel() == q.size(1));
+  }
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
               k_cache.dim() == 4 && v_cache.dim() == 4 &&
@@ -731,41 +808,42 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
     const int chunks = D / vec;
     const int nch = chunks <= 8 ? 1 : (chunks <= 16 ? 2 : 4);
     int KT = rt == 8 ? 512 : 1024;         // keeps the LDS stage under 64 KB
-    if (window > 0 && window < KT) KT = ((int)window + 31) / 32 * 32;
+    if (window > 0 && window + kf < KT) KT = ((int)window + kf + 31) / 32 * 32;
     const size_t lds_bytes =
         ((size_t)rt * KT + KT + 3 * rt + 4 * rt * 256) * 4;
     const dim3 grid(T, G, (R + rt - 1) / rt);
     const float* p1 = bias ? r1.data_ptr<float>() : nullptr;
     const float* p2 = bias ? r2.data_ptr<float>() : nullptr;
+    const float* ps = has_sinks ? sinks.data_ptr<float>() : nullptr;
     KAITO_DISPATCH_ACT(q, {
       if (rt == 8)
         launch_decode<act_t, 8>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT);
+            BS, KT, kf, ps);
       else if (rt == 4)
         launch_decode<act_t, 4>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT);
+            BS, KT, kf, ps);
       else if (rt == 2)
         launch_decode<act_t, 2>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT);
+            BS, KT, kf, ps);
       else
         launch_decode<act_t, 1>(nch, grid, lds_bytes, stream0, out, q,
             k_cache, v_cache, block_tables, token_seq, positions,
             (float)scale, (float)softcap, p1, p2, (int)window, H, G, D, V,
-            BS, KT);
+            BS, KT, kf, ps);
     });
     return;
   }
   // other sizes: one head per workgroup, one key per thread
   // keys per tile: the window when it is short, else 256
   int threads = 256;
-  if (window > 0 && window <= 64) threads = 64;
-  else if (window > 0 && window <= 128) threads = 128;
+  if (window > 0 && window + kf <= 64) threads = 64;
+  else if (window > 0 && window + kf <= 128) threads = 128;
   while (4 * threads < V) threads <<= 1;
   TORCH_CHECK(threads <= 1024, "value size too large: ", V);
   const size_t lds_bytes = ((size_t)D + 2 * threads) * 4;
@@ -778,7 +856,8 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor k_cache,
         (int)block_tables.size(1), token_seq.data_ptr<int>(),
         positions.data_ptr<int64_t>(), (float)scale, (float)softcap,
         bias ? r1.data_ptr<float>() : nullptr,
-        bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, D, V, BS);
+        bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, D, V, BS,
+        kf, has_sinks ? sinks.data_ptr<float>() : nullptr);
   });
 }
 
@@ -791,9 +870,17 @@ void window_attention_tiles(at::Tensor out, at::Tensor q, at::Tensor k_cache,
                             at::Tensor tile_seq, at::Tensor tile_qbase,
                             at::Tensor cu_seqlens, at::Tensor seq_starts,
                             double scale, double softcap, at::Tensor r1,
-                            at::Tensor r2, int64_t window) {
+                            at::Tensor r2, int64_t window, int64_t keep_first,
+                            at::Tensor sinks) {
   TORCH_CHECK(q.is_cuda() && q.dim() == 3 && q.is_contiguous() &&
               q.dtype() == at::kBFloat16);
+  TORCH_CHECK(keep_first >= 0 && keep_first < (1 << 30));
+  const int kf = window > 0 ? (int)keep_first : 0;
+  const bool has_sinks = sinks.numel() > 0;
+  if (has_sinks) {
+    KAITO_CHECK_F32(sinks);
+    TORCH_CHECK(sinks.numel() == q.size(1));
+  }
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
               k_cache.dim() == 4 && v_cache.dim() == 4 &&
@@ -829,23 +916,25 @@ void window_attention_tiles(at::Tensor out, at::Tensor q, at::Tensor k_cache,
         seq_starts.data_ptr<int>(), block_tables.data_ptr<int>(),            \
         (int)block_tables.size(1), (float)scale, (float)softcap,             \
         bias ? r1.data_ptr<float>() : nullptr,                               \
-        bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, BS);       \
+        bias ? r2.data_ptr<float>() : nullptr, (int)window, H, G, BS, kf,    \
+        has_sinks ? sinks.data_ptr<float>() : nullptr);                      \
     return;                                                                  \
   }
   KAITO_WIN_CASE(64, 64) KAITO_WIN_CASE(64, 128) KAITO_WIN_CASE(128, 64)
   KAITO_WIN_CASE(128, 128) KAITO_WIN_CASE(128, 256) KAITO_WIN_CASE(256, 128)
   KAITO_WIN_CASE(256, 256) KAITO_WIN_CASE(64, 256) KAITO_WIN_CASE(256, 64)
+  KAITO_WIN_CASE(64, 32) KAITO_WIN_CASE(128, 32)
 #undef KAITO_WIN_CASE
-  TORCH_CHECK(false, "window_attention_tiles: key/value sizes must be from "
-              "{64, 128, 256}, got ", D, "/", V);
+  TORCH_CHECK(false, "window_attention_tiles: key sizes {64, 128, 256} and "
+              "value sizes {32, 64, 128, 256}, got ", D, "/", V);
 }
 
 }  // namespace kaito
 
 TORCH_LIBRARY_FRAGMENT(kaito, m) {
-  m.def("window_attention_tiles(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor tile_seq, Tensor tile_qbase, Tensor cu_seqlens, Tensor seq_starts, float scale, float softcap, Tensor r1, Tensor r2, int window) -> ()");
-  m.def("qk_norm_cache_write(Tensor(a!) q_out, Tensor q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, float eps, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slot_mapping) -> ()");
-  m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor token_seq, Tensor positions, float scale, float softcap, Tensor r1, Tensor r2, int window) -> ()");
+  m.def("window_attention_tiles(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor tile_seq, Tensor tile_qbase, Tensor cu_seqlens, Tensor seq_starts, float scale, float softcap, Tensor r1, Tensor r2, int window, int keep_first, Tensor sinks) -> ()");
+  m.def("qk_norm_cache_write(Tensor(a!) q_out, Tensor q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, float eps, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slot_mapping, Tensor positions, Tensor inv_freq, float rot_mag, Tensor v_first, float v_lambda) -> ()");
+  m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor token_seq, Tensor positions, float scale, float softcap, Tensor r1, Tensor r2, int window, int keep_first, Tensor sinks) -> ()");
 }
 TORCH_LIBRARY_IMPL(kaito, CUDA, m) {
   m.impl("qk_norm_cache_write", &kaito::qk_norm_cache_write);
