@@ -32,11 +32,12 @@ for _g, _names in {
     "quant": "w4a16_gemv w4a16_dequant w4a16_gemm lora_shrink lora_expand",
     "comm": ("allreduce_rmsnorm one_shot_ar_rmsnorm ipc_handle ipc_open "
              "ipc_close"),
-    "mix": ("causal_conv_update gated_delta_rule rglru_scan "
+    "mix": ("causal_conv_update "
             "qk_norm_cache_write window_attention window_attention_tiles "
-            "post_norm_residual "
-            "rms_norm_cast mlstm_scan ssd_scan residual_add_norm "
+            "post_norm_residual rms_norm_cast residual_add_norm "
             "clamped_glu sigmoid_mul"),
+    "delta": "gated_delta_rule rglru_scan",
+    "decay": "mlstm_scan ssd_scan",
 }.items():
     for _n in _names.split():
         _OP_GROUP[_n] = _g

@@ -36,13 +36,15 @@ GROUPS: Dict[str, List[str]] = {
     "moe": ["bind_moe.cpp", "moe.hip"],
     "quant": ["bind_quant.cpp", "w4a16.hip", "lora.hip"],
     "comm": ["bind_comm.cpp", "allreduce_rmsnorm.hip"],
-    # stateful sequence mixers of hybrid stacks: short convolutions, gated
-    # delta rule, gated linear recurrence, scalar-decay matrix recurrences
-    # (mLSTM, state-space duality), window attention, f32 residual norms,
-    # element-wise gates (each source registers its own ops)
-    "mix": ["causal_conv.hip", "delta_rule.hip", "rglru.hip",
-            "window_attention.hip", "residual_norm.hip",
-            "decay_recurrence.hip", "gated_act.hip"],
+    # hybrid stacks (each source registers its own ops). "mix": what every
+    # hybrid design uses — short convolutions, window attention over the
+    # paged cache, f32 residual norms, element-wise gates
+    "mix": ["causal_conv.hip", "window_attention.hip", "residual_norm.hip",
+            "gated_act.hip"],
+    # gated delta rule and real-gated linear recurrence
+    "delta": ["delta_rule.hip", "rglru.hip"],
+    # scalar-decay matrix recurrences: mLSTM, state-space duality
+    "decay": ["decay_recurrence.hip"],
 }
 
 

@@ -225,3 +225,157 @@ def forward(cfg, W, tokens, streams=None):
         if streams is not None:
             streams.append(x.copy())
     return (rms(x, eps) * W["final.norm"]) @ W["head"].T
+
+
+# ---- configurations and random checkpoints for tests ---------------------
+
+def mlstm_layer(heads, dim, vdim, gate_cap=10.0, mlp=None):
+    return {"type": "mlstm", "mlp": mlp, "mixer": {
+        "heads": heads, "dim": dim, "vdim": vdim, "gate_cap": gate_cap}}
+
+
+def rot(dims, base=10000.0, scaling=None):
+    r = {"dims": dims, "base": base}
+    if scaling:
+        r["scaling"] = dict(zip(("factor", "original", "fast", "slow"),
+                                scaling))
+    return r
+
+
+def attention_mixer(heads, kv_heads, dim, vdim, conv, rot_, scale,
+                    window=None, keep_first=0, v_mix=False):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+         "conv": conv, "rot": rot_, "scale": scale}
+    if window is not None:
+        m["mask"] = {"size": window, "keep_first": keep_first}
+    if v_mix:
+        m["v_mix"] = True
+    return m
+
+
+def attention_layer(mlp=None, **kw):
+    return {"type": "attention", "mlp": mlp, "mixer": attention_mixer(**kw)}
+
+
+def parallel_layer(left, heads, vdim, state, groups, norm_groups, conv,
+                   left_scale=0.5, right_scale=0.5, mlp=None):
+    return {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": left, "left_scale": left_scale, "right_scale": right_scale,
+        "right": {"heads": heads, "vdim": vdim, "state": state,
+                  "groups": groups, "norm_groups": norm_groups,
+                  "conv": conv}}}
+
+
+def dense(ff, limit=4.0):
+    return {"kind": "dense", "ff": ff, "limit": limit}
+
+
+def make_config(layers, width, vocab, eps=1e-5):
+    return {"architecture": "Pokulorn", "layers": layers,
+            "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
+def random_weights(cfg, seed=0, slow_decay=False):
+    """bf16-representable random tensors under the checkpoint's names, as
+    float64 numpy arrays. slow_decay keeps the recurrent memories long
+    (forget gates near 1, small state-space steps) so that far-away
+    tokens still matter."""
+    import torch
+    gen = torch.Generator().manual_seed(seed)
+    W = {}
+
+    def rnd(name, *shape, std=1.0, mean=0.0):
+        t = torch.randn(*shape, generator=gen) * std + mean
+        W[name] = t.to(torch.bfloat16).double().numpy()
+
+    width = cfg["width"]
+    rnd("embed", cfg["vocab"], width)
+    rnd("final.norm", width, std=0.2, mean=1.0)
+    rnd("head", cfg["vocab"], width, std=width ** -0.5)
+
+    def attention_weights(q, a, gate, sink):
+        nq, nk, nv = (a["heads"] * a["dim"], a["kv_heads"] * a["dim"],
+                      a["kv_heads"] * a["vdim"])
+        for n, rows in (("q", nq), ("k", nk), ("v", nv)):
+            rnd(q + n, rows, width, std=width ** -0.5)
+            rnd(q + n + ".conv", rows, a["conv"], std=0.6)
+        rnd(q + "q.norm", a["dim"], std=0.3, mean=1.0)
+        rnd(q + "k.norm", a["dim"], std=0.3, mean=1.0)
+        if sink:
+            rnd(q + "sink", a["heads"], std=1.0)
+        if a.get("v_mix"):
+            W[q + "vmix"] = np.float64(
+                torch.rand((), generator=gen).to(torch.bfloat16).item())
+        if gate:
+            rnd(q + "g", a["heads"] * a["vdim"], width, std=width ** -0.5)
+        rnd(q + "o", width, a["heads"] * a["vdim"],
+            std=(a["heads"] * a["vdim"]) ** -0.5)
+
+    for i, L in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        rnd(p + "norm1", width, std=0.2, mean=1.0)
+        m = L["mixer"]
+        if L["type"] == "mlstm":
+            q = p + "mix."
+            nqk, nv = m["heads"] * m["dim"], m["heads"] * m["vdim"]
+            rnd(q + "q", nqk, width, std=width ** -0.5)
+            rnd(q + "k", nqk, width, std=width ** -0.5)
+            rnd(q + "v", nv, width, std=width ** -0.5)
+            rnd(q + "g", nv, width, std=width ** -0.5)
+            rnd(q + "i", m["heads"], width, std=2 * width ** -0.5)
+            rnd(q + "i.b", m["heads"], std=0.5)
+            rnd(q + "f", m["heads"], width, std=2 * width ** -0.5)
+            rnd(q + "f.b", m["heads"], std=0.5,
+                mean=6.0 if slow_decay else 2.0)
+            rnd(q + "norm", nv, std=0.3, mean=1.0)
+            rnd(q + "o", width, nv, std=nv ** -0.5)
+        elif L["type"] == "attention":
+            attention_weights(p + "mix.", m, gate=False, sink=True)
+        else:
+            attention_weights(p + "mix.left.", m["left"], gate=True,
+                              sink=False)
+            r, q = m["right"], p + "mix.right."
+            inner = r["heads"] * r["vdim"]
+            ch = inner + 2 * r["groups"] * r["state"]
+            rnd(q + "in", inner + ch + r["heads"], width, std=width ** -0.5)
+            rnd(q + "conv", ch, r["conv"], std=0.6)
+            rnd(q + "conv.b", ch, std=0.2)
+            rnd(q + "dt_bias", r["heads"], std=0.5,
+                mean=-4.0 if slow_decay else -1.0)
+            rnd(q + "A_log", r["heads"], std=0.5,
+                mean=-3.0 if slow_decay else 0.0)
+            rnd(q + "D", r["heads"], std=0.5, mean=1.0)
+            rnd(q + "norm", inner, std=0.3, mean=1.0)
+            rnd(q + "o", width, inner, std=inner ** -0.5)
+        if L.get("mlp") is not None:
+            q, ff = p + "mlp.", L["mlp"]["ff"]
+            rnd(p + "norm2", width, std=0.2, mean=1.0)
+            rnd(q + "gate", ff, width, std=2 * width ** -0.5)
+            rnd(q + "up", ff, width, std=2 * width ** -0.5)
+            rnd(q + "down", width, ff, std=ff ** -0.5)
+    return W
+
+
+def write_checkpoint(folder, cfg, W):
+    import json
+    import os
+
+    import torch
+    from safetensors.torch import save_file
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: torch.tensor(np.asarray(v)).to(torch.bfloat16).contiguous()
+               for k, v in W.items()},
+              os.path.join(folder, "model.safetensors"))
+    return folder
+
+
+def model_logits(cfg, W, tokens, streams=None):
+    """forward() as a float64 torch tensor (streams likewise)."""
+    import torch
+    st = [] if streams is not None else None
+    out = torch.from_numpy(forward(cfg, W, tokens, st))
+    if streams is not None:
+        streams.extend(torch.from_numpy(s) for s in st)
+    return out
