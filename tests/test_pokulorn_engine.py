@@ -303,7 +303,7 @@ def test_kept_first_token_decides_far_later(tmp_path_factory, mode):
     dropped = list(base)
     dropped[3] = (dropped[3] + 5) % cfg["vocab"]
     want_kept = P.model_logits(cfg, W, kept)[-3:]
-    assert row_err(want_kept.float(), want) > 10 * tol(mode), \
+    assert row_err(want_kept.float(), want) > 0.4, \
         "the oracle itself must depend on the kept token"
     check(last_rows(kept, sizes), want_kept, mode)
     assert row_err(last_rows(dropped, sizes), ref.double().cpu()) < 1e-6
