@@ -55,11 +55,12 @@ def parse_args():
     p.add_argument("--hybrid-compare", default=None, nargs="?", const="all",
                    metavar="SIZES",
                    help="instead of the headline workload: prefill and "
-                        "decode tokens/s of the hybrid (Gurapel) stack "
-                        "beside the sliding-window MoE transformer of equal "
-                        "size, random weights; comma-separated sizes of "
+                        "decode tokens/s of the hybrid stacks beside the "
+                        "sliding-window MoE transformer of equal size, "
+                        "random weights; comma-separated sizes of "
                         "kaito_amd.engine.hybrid_bench.SIZES (default all), "
-                        "one JSON line per size and model")
+                        "one JSON line per size and model; --hybrid-models "
+                        "picks from gurapel, pokulorn, swa-moe")
     p.add_argument("--hybrid-batch", type=int, default=32)
     p.add_argument("--hybrid-prompt", type=int, default=2048)
     p.add_argument("--hybrid-out", type=int, default=128)

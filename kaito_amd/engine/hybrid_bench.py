@@ -1,8 +1,9 @@
-"""Prefill and decode throughput of the hybrid (Gurapel) stack beside the
-engine's closest homogeneous model at equal size: a sliding-window GQA
-transformer with the same MoE feed-forward (the gpt-oss class without
-sinks). Random weights, synthetic tokens; both models run through the
-same LLMEngine (scheduler, paged cache, hipGraph decode).
+"""Prefill and decode throughput of the hybrid stacks (Gurapel, Pokulorn)
+beside each other and beside the engine's closest homogeneous model at
+equal size: a sliding-window GQA transformer with the same MoE
+feed-forward (the gpt-oss class without sinks). Random weights, synthetic
+tokens; all models run through the same LLMEngine (scheduler, paged
+cache, hipGraph decode).
 
 Used by `bench.py --hybrid-compare`; prints one JSON line per
 (size, model).
@@ -48,6 +49,40 @@ def hybrid_config(name: str, z: dict, max_pos: int):
         "architecture": "Gurapel", "embedding": {"scale": 1.0},
         "layers": layers, "max_positions": max_pos, "norm": {"eps": 1e-5},
         "vocab": z["vocab"], "width": z["width"]}, name=f"gurapel-{name}")
+
+
+def pokulorn_config(name: str, z: dict, max_pos: int):
+    """The pre-norm hybrid at the sizes of `z`: layers cycle matrix
+    memory, windowed attention, attention beside a state-space mixer. The
+    recurrent states match the Gurapel stack's (one dim x dim matrix per
+    head); the dense feed-forward is as wide as the MoE's active experts
+    together."""
+    from ..models.hybrid_config import pokulorn_model_config
+    ff = {"kind": "dense", "ff": z["ff"] * z["top"], "limit": 7.0}
+    rot = {"base": 10000.0, "dims": z["dim"] // 2,
+           "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0,
+                       "slow": 1.0}}
+    mem = {"type": "mlstm", "mlp": ff, "mixer": {
+        "heads": z["heads"], "dim": z["dim"], "vdim": z["dim"],
+        "gate_cap": 15.0}}
+    att = {"type": "attention", "mlp": ff, "mixer": {
+        "heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"],
+        "vdim": z["dim"], "conv": 4, "rot": rot, "scale": z["dim"] ** -0.5,
+        "mask": {"size": z["window"], "keep_first": 64}, "v_mix": True}}
+    par = {"type": "parallel", "mlp": ff, "mixer": {
+        "left": {"heads": z["heads"], "kv_heads": z["kv_heads"],
+                 "dim": z["dim"], "vdim": z["dim"], "conv": 4, "rot": rot,
+                 "scale": z["dim"] ** -0.5,
+                 "mask": {"size": z["window"], "keep_first": 0}},
+        "right": {"heads": z["width"] // 64, "vdim": 64, "state": 128,
+                  "groups": z["kv_heads"], "norm_groups": z["kv_heads"],
+                  "conv": 4},
+        "left_scale": 0.5, "right_scale": 0.5}}
+    layers = [(mem, att, par)[i % 3] for i in range(z["layers"])]
+    return pokulorn_model_config({
+        "architecture": "Pokulorn", "layers": layers,
+        "max_positions": max_pos, "norm": {"eps": 1e-5},
+        "vocab": z["vocab"], "width": z["width"]}, name=f"pokulorn-{name}")
 
 
 def transformer_config(name: str, z: dict, max_pos: int):
@@ -118,8 +153,8 @@ def run(sizes: List[str], batch: int, prompt: int, out_tokens: int,
         z = SIZES[name]
         max_pos = prompt + out_tokens + 16
         for kind in models:
-            mcfg = hybrid_config(name, z, max_pos) if kind == "gurapel" \
-                else transformer_config(name, z, max_pos)
+            mcfg = {"gurapel": hybrid_config, "pokulorn": pokulorn_config,
+                    "swa-moe": transformer_config}[kind](name, z, max_pos)
             pre, dec = _measure(mcfg, batch, prompt, out_tokens, eager)
             row = {"bench": "hybrid-compare", "size": name, "model": kind,
                    "batch": batch, "prompt_tokens": prompt,

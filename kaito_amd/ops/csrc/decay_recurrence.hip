@@ -24,12 +24,13 @@
 // scan, one thread per (chunk, head), adds and maxima only; exponentials
 // token-parallel] -> recurrence -> epilogue (token-parallel).
 //
-// Recurrence kernel: one single-wave workgroup per (chunk, head, group of 16
-// state columns); lane (column, part) keeps DP rows of its column in
-// registers, so a token costs 2 DP FMAs per lane and one 4-lane butterfly.
+// Recurrence kernel: one single-wave workgroup per (chunk, head, group of 8
+// or 16 state columns); lane (column, part) keeps DP rows of its column in
+// registers, so a token costs 3 DP VALU operations per lane and one 4- or
+// 8-lane butterfly.
 // Token tiles are double-buffered: the next tile's global loads are issued
 // before the current tile is consumed and parked in LDS afterwards. k and q
-// rows are zero-padded to 4 DP in LDS so the inner loop is unconditional
+// rows are zero-padded to DP * parts in LDS so the inner loop is unconditional
 // float4 reads. A chunk that starts at position 0 starts from S = 0 whatever
 // its slot held; slots < 0 are padding and skipped.
 #include "mix_common.h"
@@ -39,10 +40,10 @@ namespace kaito {
 namespace {
 
 constexpr int RTT = 8;          // tokens per tile
-constexpr int RPARTS = 4;       // lanes per state column
-constexpr int RVB = 64 / RPARTS;  // state columns per wave
 
-template <typename T, int DP>
+// RPARTS lanes share one state column (DP rows each); a wave covers
+// RVB = 64 / RPARTS columns
+template <typename T, int DP, int RPARTS>
 __global__ __launch_bounds__(64) void decay_recurrence_kernel(
     float* __restrict__ o,                    // [T, H, V]
     float* __restrict__ o_n,                  // [T, H] or null
@@ -55,6 +56,7 @@ __global__ __launch_bounds__(64) void decay_recurrence_kernel(
     const int* __restrict__ cu, const int* __restrict__ slots,
     const int* __restrict__ starts, const int G, const int D, const int H,
     const int V, const float q_scale) {
+  constexpr int RVB = 64 / RPARTS;
   constexpr int DPAD = DP * RPARTS;
   // each part's DP-slice is followed by 4 floats of padding: lanes of
   // different parts read their slices in the same instruction, and slices a
@@ -88,19 +90,43 @@ __global__ __launch_bounds__(64) void decay_recurrence_kernel(
     S[i] = (carried && live && d < D) ? sp[(int64_t)d * sp_stride] : 0.0f;
   }
 
+  // fetch() issues every load of a tile unconditionally (rows and columns
+  // clamped into range) so that none of them waits for another; what lies
+  // outside the tile is zeroed when the registers are parked in LDS
   float rk[KQN], rq[KQN], rv[VN], rc = 0.f;
+  int fetched_nt = 0;
   auto fetch = [&](int t0) {
     const int nt = min(RTT, r1 - t0);
+    fetched_nt = nt;
+#pragma unroll
+    for (int i = 0; i < KQN; i++) {
+      const int e = tid + i * 64;
+      const int tt = min(e / DPAD, nt - 1), d = min(e % DPAD, D - 1);
+      rk[i] = act_ld(k + (int64_t)(t0 + tt) * k_s0 + (int64_t)g * k_s1 + d);
+      rq[i] = act_ld(q + (int64_t)(t0 + tt) * q_s0 + (int64_t)g * q_s1 + d);
+    }
+#pragma unroll
+    for (int i = 0; i < VN; i++) {
+      const int e = tid + i * 64;
+      const int tt = min(e / RVB, nt - 1);
+      const int c = min((int)blockIdx.z * RVB + e % RVB, V - 1);
+      rv[i] = act_ld(v + (int64_t)(t0 + tt) * v_s0 + (int64_t)h * v_s1 + c);
+    }
+    if (tid < 2 * RTT) {
+      const int tt = min(tid >> 1, nt - 1);
+      rc = ((tid & 1) ? take : keep)[(int64_t)(t0 + tt) * H + h];
+    }
+  };
+  auto park = [&](float* buf) {
+    const int nt = fetched_nt;
 #pragma unroll
     for (int i = 0; i < KQN; i++) {
       const int e = tid + i * 64;
       const int tt = e / DPAD, d = e % DPAD;
       const bool ok = tt < nt && d < D;
-      rk[i] = ok ? act_ld(k + (int64_t)(t0 + tt) * k_s0 + (int64_t)g * k_s1 + d)
-                 : 0.f;
-      rq[i] = ok ? act_ld(q + (int64_t)(t0 + tt) * q_s0 + (int64_t)g * q_s1 + d)
-                       * q_scale
-                 : 0.f;
+      const int dd = (d / DP) * DPS + d % DP;
+      buf[tt * ROW + dd] = ok ? rk[i] : 0.f;
+      buf[tt * ROW + KROW + dd] = ok ? rq[i] * q_scale : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < VN; i++) {
@@ -108,34 +134,14 @@ __global__ __launch_bounds__(64) void decay_recurrence_kernel(
       const int tt = e / RVB, c = blockIdx.z * RVB + e % RVB;
       float val = 0.f;
       if (tt < nt) {
-        if (c < V)
-          val = act_ld(v + (int64_t)(t0 + tt) * v_s0 + (int64_t)h * v_s1 + c);
-        else if (state_n != nullptr && c == V)
-          val = 1.0f;
+        if (c < V) val = rv[i];
+        else if (state_n != nullptr && c == V) val = 1.0f;
       }
-      rv[i] = val;
+      buf[tt * ROW + 2 * KROW + e % RVB] = val;
     }
-    if (tid < 2 * RTT) {
-      const int tt = tid >> 1;
-      rc = tt < nt ? ((tid & 1) ? take : keep)[(int64_t)(t0 + tt) * H + h]
-                   : 0.f;
-    }
-  };
-  auto park = [&](float* buf) {
-#pragma unroll
-    for (int i = 0; i < KQN; i++) {
-      const int e = tid + i * 64;
-      const int tt = e / DPAD, d = e % DPAD;
-      const int dd = (d / DP) * DPS + d % DP;
-      buf[tt * ROW + dd] = rk[i];
-      buf[tt * ROW + KROW + dd] = rq[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VN; i++) {
-      const int e = tid + i * 64;
-      buf[(e / RVB) * ROW + 2 * KROW + e % RVB] = rv[i];
-    }
-    if (tid < 2 * RTT) buf[(tid >> 1) * ROW + 2 * KROW + RVB + (tid & 1)] = rc;
+    if (tid < 2 * RTT)
+      buf[(tid >> 1) * ROW + 2 * KROW + RVB + (tid & 1)] =
+          (tid >> 1) < nt ? rc : 0.f;
   };
 
   fetch(r0);
@@ -149,25 +155,28 @@ __global__ __launch_bounds__(64) void decay_recurrence_kernel(
     const float* buf = lds[cur];
     for (int tt = 0; tt < nt; tt++) {
       const float* lk = buf + tt * ROW + part * DPS;
-      const float* lq = lk + KROW;
+      // all LDS reads of the token first, then three passes of mutually
+      // independent instructions (a lone wave on a SIMD has nothing else
+      // to cover the latency of back-to-back dependent ones)
+      float4_t k4[DP / 4], q4[DP / 4];
+#pragma unroll
+      for (int i = 0; i < DP / 4; i++) {
+        k4[i] = *reinterpret_cast<const float4_t*>(lk + 4 * i);
+        q4[i] = *reinterpret_cast<const float4_t*>(lk + KROW + 4 * i);
+      }
       const float kp = buf[tt * ROW + 2 * KROW + RVB];
       const float u = buf[tt * ROW + 2 * KROW + RVB + 1] *
                       buf[tt * ROW + 2 * KROW + jl];
-      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      float w[DP];
 #pragma unroll
-      for (int i = 0; i < DP; i += 4) {
-        const float4_t k4 = *reinterpret_cast<const float4_t*>(lk + i);
-        const float4_t q4 = *reinterpret_cast<const float4_t*>(lq + i);
-        S[i] = kp * S[i] + k4[0] * u;
-        S[i + 1] = kp * S[i + 1] + k4[1] * u;
-        S[i + 2] = kp * S[i + 2] + k4[2] * u;
-        S[i + 3] = kp * S[i + 3] + k4[3] * u;
-        a0 += S[i] * q4[0];
-        a1 += S[i + 1] * q4[1];
-        a2 += S[i + 2] * q4[2];
-        a3 += S[i + 3] * q4[3];
-      }
-      const float oj = group_reduce_sum<RPARTS>((a0 + a1) + (a2 + a3));
+      for (int i = 0; i < DP; i++) w[i] = k4[i / 4][i % 4] * u;
+#pragma unroll
+      for (int i = 0; i < DP; i++) S[i] = kp * S[i] + w[i];
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < DP; i++) acc[i % 4] += S[i] * q4[i / 4][i % 4];
+      const float oj =
+          group_reduce_sum<RPARTS>((acc[0] + acc[1]) + (acc[2] + acc[3]));
       if (part == 0) {
         if (j < V) o[((int64_t)(t0 + tt) * H + h) * V + j] = oj;
         else if (ncol) o_n[(int64_t)(t0 + tt) * H + h] = oj;
@@ -197,10 +206,11 @@ struct RecurrenceArgs {
   float q_scale;
 };
 
-template <typename T, int DP>
+template <typename T, int DP, int RPARTS>
 void launch_recurrence_dp(const RecurrenceArgs& a, hipStream_t stream) {
+  constexpr int RVB = 64 / RPARTS;
   const int cols = a.V + (a.state_n ? 1 : 0);
-  hipLaunchKernelGGL((decay_recurrence_kernel<T, DP>),
+  hipLaunchKernelGGL((decay_recurrence_kernel<T, DP, RPARTS>),
       dim3(a.B, a.H, (cols + RVB - 1) / RVB), dim3(64), 0, stream, a.o, a.o_n,
       (const T*)a.q, a.q_s0, a.q_s1, (const T*)a.k, a.k_s0, a.k_s1,
       (const T*)a.v, a.v_s0, a.v_s1, a.keep, a.take, a.state, a.state_n, a.cu,
@@ -209,12 +219,13 @@ void launch_recurrence_dp(const RecurrenceArgs& a, hipStream_t stream) {
 
 template <typename T>
 void launch_recurrence(const RecurrenceArgs& a, hipStream_t stream) {
-  const int need = (a.D + RPARTS - 1) / RPARTS;
-  if (need <= 4) launch_recurrence_dp<T, 4>(a, stream);
-  else if (need <= 8) launch_recurrence_dp<T, 8>(a, stream);
-  else if (need <= 16) launch_recurrence_dp<T, 16>(a, stream);
-  else if (need <= 32) launch_recurrence_dp<T, 32>(a, stream);
-  else if (need <= 64) launch_recurrence_dp<T, 64>(a, stream);
+  // few rows per lane keep the register count low enough for several
+  // waves per SIMD; eight lanes per column also double the number of waves
+  if (a.D <= 16) launch_recurrence_dp<T, 4, 4>(a, stream);
+  else if (a.D <= 32) launch_recurrence_dp<T, 8, 4>(a, stream);
+  else if (a.D <= 64) launch_recurrence_dp<T, 8, 8>(a, stream);
+  else if (a.D <= 128) launch_recurrence_dp<T, 16, 8>(a, stream);
+  else if (a.D <= 256) launch_recurrence_dp<T, 32, 8>(a, stream);
   else TORCH_CHECK(false, "state rows per head must be <= 256, got ", a.D);
 }
 
