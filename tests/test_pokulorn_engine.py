@@ -72,22 +72,22 @@ def config_c():
     # value 32 / 64; windows past two key tiles with kept tokens between
     return P.make_config([
         P.attention_layer(heads=2, kv_heads=1, dim=64, vdim=32, conv=3,
-                          rot_=P.rot(64, base=20000.0,
-                                     scaling=(4.0, 64, 32.0, 1.0)),
+                          rot_=P.rot(64, base=50000.0,
+                                     scaling=(8.0, 64, 32.0, 1.0)),
                           scale=0.125, window=19, keep_first=5, v_mix=True,
-                          mlp=P.dense(64, 1.0)),
-        P.mlstm_layer(heads=2, dim=32, vdim=32, gate_cap=12.0),
+                          mlp=P.dense(64, 2.0)),
+        P.mlstm_layer(heads=2, dim=32, vdim=32, gate_cap=9.0),
         P.attention_layer(heads=2, kv_heads=1, dim=128, vdim=32, conv=3,
-                          rot_=P.rot(32, base=20000.0), scale=0.09,
-                          window=40, keep_first=20, v_mix=True,
-                          mlp=P.dense(64, 1.0)),
+                          rot_=P.rot(32, base=30000.0), scale=0.09,
+                          window=44, keep_first=23, v_mix=True,
+                          mlp=P.dense(64, 2.0)),
         P.parallel_layer(
             P.attention_mixer(heads=2, kv_heads=2, dim=64, vdim=64, conv=4,
                               rot_=P.rot(32, base=10000.0,
                                          scaling=(2.0, 128, 32.0, 1.0)),
                               scale=0.125),
-            heads=4, vdim=32, state=16, groups=2, norm_groups=2, conv=4,
-            left_scale=0.6, right_scale=0.5, mlp=P.dense(96, 1.0)),
+            heads=4, vdim=32, state=16, groups=4, norm_groups=1, conv=3,
+            left_scale=0.8, right_scale=0.3, mlp=P.dense(96, 2.0)),
     ], width=128, vocab=64)
 
 

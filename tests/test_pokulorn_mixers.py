@@ -55,7 +55,7 @@ def f64(t):
 
 @pytest.mark.parametrize("rot", [
     P.rot(16), P.rot(8, base=500.0),
-    P.rot(32, base=20000.0, scaling=(4.0, 64, 32.0, 1.0)),
+    P.rot(32, base=40000.0, scaling=(4.0, 64, 32.0, 1.0)),
     P.rot(16, base=10000.0, scaling=(2.0, 4096, 16.0, 2.0)),
     P.rot(64, base=1e6, scaling=(16.0, 128, 32.0, 1.0))])
 def test_rotary_frequencies(rot):
@@ -246,7 +246,7 @@ def test_sink_counts_once_unscaled(mode):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,G,D,V,window,keep,sink", [
-    (4, 1, 64, 32, 40, 20, True), (2, 2, 64, 64, 0, 0, False),
+    (4, 1, 64, 32, 48, 24, True), (2, 2, 64, 64, 0, 0, False),
     (2, 1, 128, 32, 70, 33, True), (2, 2, 64, 128, 33, 64, False),
     (2, 1, 64, 32, 100, 5, True)])
 def test_tiled_prompt_kernel_window_first_tokens_sink(H, G, D, V, window,
@@ -291,7 +291,7 @@ def plain_mlstm(q, k, v, gate, ipre, fpre, norm_w, cap, eps):
 
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("H,D,V,cap", [(2, 16, 24, 15.0), (3, 8, 8, 4.0),
-                                       (1, 48, 48, 12.0), (2, 10, 17, 8.0),
+                                       (1, 56, 40, 11.0), (2, 10, 17, 8.0),
                                        (1, 128, 64, 20.0), (4, 24, 15, 2.0)])
 def test_mlstm_portions_and_stale_slots(mode, H, D, V, cap):
     dev, dt = mode
