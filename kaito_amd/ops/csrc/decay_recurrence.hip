@@ -21,7 +21,7 @@
 //               y = o + D x, times silu(z), RMS norm in equal parts, weight.
 //
 // Launches: gate/step activations (token-parallel) -> [mlstm: running-maximum
-// scan, one thread per (chunk, head), adds and maxima only; exponentials
+// scan, one wave per (chunk, head) over (max, +) pairs; exponentials
 // token-parallel] -> recurrence -> epilogue (token-parallel).
 //
 // Recurrence kernel: one single-wave workgroup per (chunk, head, group of 8
@@ -247,28 +247,51 @@ __global__ void mlstm_gate_kernel(
   gf[e] = log_sigmoid_f(cap * tanhf(fpre[(int64_t)t * f_s0 + h] * inv));
 }
 
-// m after every token and m before it; the only serial part
-__global__ void mlstm_max_scan_kernel(
+// m after every token and m before it. The step m -> max(m + f, i) is a
+// pair (A, B) acting as m -> max(m + A, B); pairs compose associatively:
+// (A1, B1) then (A2, B2) = (A1 + A2, max(B1 + A2, B2)). One wave per
+// (chunk, head): every lane folds a contiguous run of tokens into a pair,
+// a shuffle scan over the 64 pairs gives each lane the m it starts from,
+// and a second pass over the run writes the values.
+__global__ __launch_bounds__(64) void mlstm_max_scan_kernel(
     float* __restrict__ m_after, float* __restrict__ m_before,   // [T, H]
     const float* __restrict__ gi, const float* __restrict__ gf,
     float* __restrict__ state_m,                                 // [slots, H]
     const int* __restrict__ cu, const int* __restrict__ slots,
-    const int* __restrict__ starts, const int B, const int H) {
-  const int e = blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= B * H) return;
-  const int b = e / H, h = e % H;
+    const int* __restrict__ starts, const int H) {
+  const int b = blockIdx.x / H, h = blockIdx.x % H;
+  const int lane = threadIdx.x;
   const int slot = slots[b];
   const int r0 = cu[b], r1 = cu[b + 1];
   if (slot < 0 || r1 <= r0) return;
-  float m = starts[b] > 0 ? state_m[(int64_t)slot * H + h] : 0.0f;
-#pragma unroll 8
-  for (int t = r0; t < r1; t++) {
+  const float m0 = starts[b] > 0 ? state_m[(int64_t)slot * H + h] : 0.0f;
+  const int run = (r1 - r0 + 63) / 64;
+  const int s0 = min(r0 + lane * run, r1), s1 = min(s0 + run, r1);
+  float A = 0.0f, B = -INFINITY;
+  for (int t = s0; t < s1; t++) {
+    const int64_t at = (int64_t)t * H + h;
+    const float f = gf[at];
+    A += f;
+    B = fmaxf(B + f, gi[at]);
+  }
+  // inclusive scan of the pairs, earlier lanes on the left
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const float Al = __shfl_up(A, off, 64), Bl = __shfl_up(B, off, 64);
+    if (lane >= off) {
+      B = fmaxf(Bl + A, B);
+      A = Al + A;
+    }
+  }
+  const float Ap = __shfl_up(A, 1, 64), Bp = __shfl_up(B, 1, 64);
+  float m = lane == 0 ? m0 : fmaxf(m0 + Ap, Bp);
+  for (int t = s0; t < s1; t++) {
     const int64_t at = (int64_t)t * H + h;
     m_before[at] = m;
     m = fmaxf(gf[at] + m, gi[at]);
     m_after[at] = m;
   }
-  state_m[(int64_t)slot * H + h] = m;
+  if (lane == 63) state_m[(int64_t)slot * H + h] = fmaxf(m0 + A, B);
 }
 
 // in place: gf <- keep, gi <- take, m_before <- exp(-m)
@@ -413,10 +436,10 @@ void mlstm_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v,
   hipLaunchKernelGGL(mlstm_gate_kernel, dim3((n + 255) / 256), dim3(256), 0,
       stream, gi, gf, ipre.data_ptr<float>(), ipre.stride(0),
       fpre.data_ptr<float>(), fpre.stride(0), n, H, (float)cap);
-  hipLaunchKernelGGL(mlstm_max_scan_kernel, dim3((B * H + 63) / 64), dim3(64),
-      0, stream, m_after, m_before, gi, gf, state_m.data_ptr<float>(),
+  hipLaunchKernelGGL(mlstm_max_scan_kernel, dim3(B * H), dim3(64), 0, stream,
+      m_after, m_before, gi, gf, state_m.data_ptr<float>(),
       cu_seqlens.data_ptr<int>(), state_slots.data_ptr<int>(),
-      seq_starts.data_ptr<int>(), B, H);
+      seq_starts.data_ptr<int>(), H);
   hipLaunchKernelGGL(mlstm_coef_kernel, dim3((n + 255) / 256), dim3(256), 0,
       stream, gi, gf, m_after, m_before, n);
   RecurrenceArgs a{o.data_ptr<float>(), o_n.data_ptr<float>(), q.data_ptr(),

@@ -322,6 +322,52 @@ def test_mlstm_portions_and_stale_slots(mode, H, D, V, cap):
 
 
 @pytest.mark.parametrize("mode", MODES)
+def test_mlstm_long_chunks_beside_short(mode):
+    """Chunks of several hundred tokens (the running maximum is scanned in
+    parallel runs inside a chunk) beside a single-token chunk; input gates
+    that jump so that the maximum is reset in the middle of runs."""
+    dev, dt = mode
+    H, D, V, cap = 2, 8, 12, 10.0
+    lens = [333, 1, 130]
+    r = lambda *s: torch.randn(*s).to(dt)  # noqa: E731
+    norm_w = torch.randn(H * V)
+    seqs, want = [], []
+    for n in lens:
+        ipre = torch.randn(n, H) * 4
+        ipre[torch.rand(n, H) < 0.03] += 25.0
+        s = (r(n, H, D), r(n, H, D), r(n, H, V), r(n, H, V), ipre,
+             torch.randn(n, H) * 2 + 3)
+        seqs.append(s)
+        want.append(plain_mlstm(*(f64(t) for t in s), f64(norm_w), cap,
+                                1e-5))
+    sc = torch.full((3, H, D, V), 1.0, device=dev)
+    sn = torch.full((3, H, D), 1.0, device=dev)
+    sm = torch.full((3, H), -3.0, device=dev)
+    got = [[] for _ in lens]
+    for cut in ((0, 200), (200, 400)):
+        parts_in, lens_now, starts, slots, owner = [], [], [], [], []
+        for i, n in enumerate(lens):
+            a, b = min(cut[0], n), min(cut[1], n)
+            if b > a:
+                parts_in.append([t[a:b] for t in seqs[i]])
+                lens_now.append(b - a)
+                starts.append(a)
+                slots.append(i)
+                owner.append(i)
+        cat = [torch.cat([p[j] for p in parts_in]).to(dev) for j in range(6)]
+        cu, sl, st, _, _ = layout(dev, lens_now, starts, slots)
+        out = ops.mlstm_scan(cat[0], cat[1], cat[2], cat[3], cat[4], cat[5],
+                             norm_w.to(dev), sc, sn, sm, cu, sl, st, cap,
+                             D ** -0.5, 1e-5)
+        row = 0
+        for i, n in zip(owner, lens_now):
+            got[i].append(out[row:row + n])
+            row += n
+    for g, w in zip(got, want):
+        close(torch.cat(g), w, dt, slack=3)
+
+
+@pytest.mark.parametrize("mode", MODES)
 def test_mlstm_running_maximum_starts_at_zero(mode):
     """Strongly negative input gates at the start: with the maximum
     starting at 0 (not at minus infinity) the first read-outs are divided
