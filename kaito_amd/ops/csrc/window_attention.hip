@@ -923,7 +923,7 @@ void window_attention_tiles(at::Tensor out, at::Tensor q, at::Tensor k_cache,
   KAITO_WIN_CASE(64, 64) KAITO_WIN_CASE(64, 128) KAITO_WIN_CASE(128, 64)
   KAITO_WIN_CASE(128, 128) KAITO_WIN_CASE(128, 256) KAITO_WIN_CASE(256, 128)
   KAITO_WIN_CASE(256, 256) KAITO_WIN_CASE(64, 256) KAITO_WIN_CASE(256, 64)
-  KAITO_WIN_CASE(64, 32) KAITO_WIN_CASE(128, 32)
+  KAITO_WIN_CASE(64, 32) KAITO_WIN_CASE(128, 32) KAITO_WIN_CASE(256, 32)
 #undef KAITO_WIN_CASE
   TORCH_CHECK(false, "window_attention_tiles: key sizes {64, 128, 256} and "
               "value sizes {32, 64, 128, 256}, got ", D, "/", V);
