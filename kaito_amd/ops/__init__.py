@@ -588,8 +588,8 @@ def residual_add_norm(x32, y, w, eps: float, out_dtype, y2=None,
     if x32.is_cuda:
         h = torch.empty(x32.shape, dtype=out_dtype, device=x32.device) \
             if w is not None else x32
-        _K.residual_add_norm(x32, h, y, _none(y2, y) if y2 is None else y2,
-                             _none(w, y), s1, s2, eps)
+        _K.residual_add_norm(x32, h, y, _none(y2, y), _none(w, y), s1, s2,
+                             eps)
         return h if w is not None else None
     return torch_ref.residual_add_norm(x32, y, w, eps, out_dtype, y2, s1, s2)
 

@@ -83,7 +83,7 @@ def rotate(x, cos, sin):
 
 
 def attention(h, W, pre, mx, eps, v_first=None, mix_values=False,
-              sink=True, gate=False, want=None):
+              sink=True, gate=False):
     """Softmax attention with short convolutions, per-head q/k norm,
     partial rotation, an optional window that keeps the first tokens, an
     optional sink in the denominator, optional mixing with another
